@@ -1,0 +1,167 @@
+/*
+ * mi_moe.h -- C ABI of the MI355X (gfx950) quantized mixture-of-experts block.
+ *
+ * One call, mi_moe_forward, replaces the ~25 mlx-sys dispatches an mlx-rs Module
+ * makes for a sparse MoE layer (router Linear, softmax, argpartition, take_along_axis,
+ * renormalise, argsort x2, take, gather_qmm x3, silu, multiply, unsort, multiply,
+ * sum).  Stage-level entry points expose each primitive family on its own so that
+ * each has an individually testable counterpart.
+ *
+ * Conventions follow what mlx-rs expects from mlx-sys:
+ *  - every entry point returns int: 0 = success, non-zero = failure
+ *    (mlx-rs/src/utils/mod.rs:13-14, mlx-rs/src/utils/guard.rs:20-49);
+ *  - the message of the last failure is kept per thread and can also be delivered to
+ *    a registered handler (mlx-rs/src/error.rs:226-280 installs such a handler through
+ *    mlx_set_error_handler and stores the text in a thread-local slot);
+ *  - no exception or unwinding crosses the boundary; on failure outputs are untouched;
+ *  - arrays are row-major and contiguous (an mlx-rs Array after eval,
+ *    mlx-rs/src/array/mod.rs:384-403); bfloat16 is passed as raw uint16_t, packed
+ *    weights and indices as uint32_t, sizes as int64_t; every pointer is DEVICE memory
+ *    unless the comment says host, and must be 16-byte aligned;
+ *  - calls are asynchronous on the hipStream_t passed as `void* stream` (NULL = the
+ *    default stream): the analogue of MLX's lazy evaluation, the caller synchronises
+ *    where mlx-rs would call eval (mlx-rs/src/transforms/mod.rs:66-92);
+ *  - the library keeps no input pointer after a call returns except the weight
+ *    pointers registered with mi_moe_create; one handle is used by one host thread at
+ *    a time (MLX itself is not thread safe, .github/workflows/validate.yml:46).
+ *
+ * Weight format = MLX "affine" quantisation (mlx-rs/src/ops/quantization.rs:31-47,
+ * 85-87, 306-309): element c of a row lives in uint32 word c/(32/bits) at bit
+ * (c mod (32/bits))*bits; w_hat = scale*q + bias with one bf16 (scale, bias) per
+ * group_size consecutive elements of the row.
+ */
+#ifndef MI_MOE_H
+#define MI_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mi_moe_s *mi_moe_handle;
+
+typedef enum {
+  MI_MOE_SCORE_SOFTMAX_THEN_TOPK_RENORM = 0, /* Qwen3-MoE, norm_topk_prob = true  */
+  MI_MOE_SCORE_SOFTMAX_THEN_TOPK = 1,        /* Qwen3-MoE, norm_topk_prob = false */
+  MI_MOE_SCORE_TOPK_THEN_SOFTMAX = 2         /* Mixtral: softmax over the selected logits */
+} mi_moe_score_mode;
+
+typedef struct {
+  int32_t hidden;       /* H, multiple of group_size */
+  int32_t n_experts;    /* E, 1..512 */
+  int32_t top_k;        /* k, 1..min(E,32) */
+  int32_t intermediate; /* I, multiple of group_size */
+  int32_t bits;         /* 4 or 8 */
+  int32_t group_size;   /* 64 */
+  int32_t score_mode;   /* mi_moe_score_mode */
+} mi_moe_config;
+
+/* one bank of E quantized matrices, the layout mlx-rs's QuantizedLinear holds per
+ * matrix (mlx-rs/src/nn/quantized.rs:254-279: inner.weight, scales, biases) with a
+ * leading expert axis */
+typedef struct {
+  const uint32_t *w;      /* [E, N, K*bits/32] */
+  const uint16_t *scales; /* bf16 [E, N, K/group_size] */
+  const uint16_t *biases; /* bf16 [E, N, K/group_size] */
+} mi_moe_qmat;
+
+typedef struct {
+  const uint16_t *router_w; /* bf16 [E, H]: bias-free Linear, mlx-rs/src/nn/linear.rs:84-96 */
+  const float *router_bias; /* f32 [E] added to the logits before the bf16 round, or NULL */
+  mi_moe_qmat gate, up;     /* N = I, K = H */
+  mi_moe_qmat down;         /* N = H, K = I */
+} mi_moe_weights;
+
+/* optional routing outputs of mi_moe_forward; any member may be NULL */
+typedef struct {
+  uint32_t *topk_idx; /* [T, k] expert ids, slot 0 = best, ties -> lower id */
+  uint16_t *topk_w;   /* bf16 [T, k] scores */
+  uint32_t *counts;   /* [E] pairs per expert */
+  uint32_t *offsets;  /* [E+1] exclusive scan of counts */
+  uint32_t *perm;     /* [P] pair index t*k+s of sorted position r (stable by expert) */
+  uint32_t *inv_perm; /* [P] sorted position of pair t*k+s */
+} mi_moe_debug_out;
+
+/* ---- errors (replaces mlx_set_error_handler + the LAST_MLX_ERROR slot,
+ * mlx-rs/src/error.rs:226-280) ---- */
+const char *mi_moe_last_error(void); /* thread-local, never NULL */
+void mi_moe_set_error_handler(void (*handler)(const char *msg, void *data), void *data,
+                              void (*dtor)(void *data));
+
+/* ---- the block (replaces the op sequence a Module<&Array>::forward would issue;
+ * forward contract mlx-rs/src/module/module.rs:28-50, dense sibling
+ * mlx-lm/src/models/qwen3.rs:204-255, call site :321-324) ---- */
+int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_moe_handle *out);
+int mi_moe_destroy(mi_moe_handle h);
+int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *bytes);
+/* x: bf16 [T, H] -> out: bf16 [T, H].  workspace: device memory of at least
+ * mi_moe_workspace_size(cfg, T) bytes, 256-byte aligned, contents irrelevant. */
+int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
+                   void *workspace, size_t workspace_bytes, const mi_moe_debug_out *dbg,
+                   void *stream);
+
+/* ---- R1-R4 router: gate Linear + softmax(precise) + argpartition top-k +
+ * take_along_axis + renormalise (mlx_matmul, mlx_softmax_axis, mlx_argpartition_axis,
+ * mlx_take_along_axis, mlx_sum_axis, mlx_divide; mlx-rs/src/ops/arithmetic.rs:577-603,
+ * 1291-1327, ops/sort.rs:211-260, ops/indexing/mod.rs:433-453).
+ * logits_out (bf16 [T,E]) may be NULL.  workspace >= mi_moe_route_workspace_size. */
+int mi_moe_route_workspace_size(int32_t n_experts, int64_t T, size_t *bytes);
+int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *router_bias,
+                 int64_t T, int32_t hidden, int32_t n_experts, int32_t top_k,
+                 int32_t score_mode, uint32_t *topk_idx, uint16_t *topk_w,
+                 uint16_t *logits_out, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- R5 dispatch: stable sort of the P = T*k pairs by expert (mlx_argsort x2,
+ * mlx_floor_divide, mlx_take; mlx-rs/src/ops/sort.rs:75-109).  Every output except
+ * perm may be NULL.  workspace >= mi_moe_dispatch_workspace_size. */
+int mi_moe_dispatch_workspace_size(int32_t n_experts, int64_t P, size_t *bytes);
+int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts,
+                    uint32_t *counts, uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- R6 gather_qmm (mlx_gather_qmm, mlx-rs/src/ops/quantization.rs:160-230):
+ * for j < n_idx: y[j] (M x N) = x[lhs[j]] (M x K) . dequantize(w[rhs[j]])^T.
+ * x: bf16 [x_batch, M, K]; w: [E, N, K*bits/32]; y: bf16 [n_idx, M, N].
+ * lhs_indices NULL = identity (j), as an absent mlx_array; rhs_indices required.
+ * transpose must be non-zero (the layout every mlx-lm switch layer uses);
+ * sorted_indices is a hint, results do not depend on it.
+ * workspace >= mi_moe_gather_qmm_workspace_size. */
+int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M, size_t *bytes);
+int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                      const uint16_t *biases, const uint32_t *lhs_indices,
+                      const uint32_t *rhs_indices, int64_t n_idx, int64_t x_batch, int32_t M,
+                      int32_t N, int32_t K, int32_t n_experts, int32_t transpose,
+                      int32_t group_size, int32_t bits, int32_t sorted_indices, uint16_t *y,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- R7 silu(gate) * up on bf16 arrays (mlx_sigmoid + mlx_multiply x2,
+ * mlx-rs/src/nn/activation.rs:142-144,876-880).  The block itself fuses this into
+ * the gate/up product; this entry point is the stand-alone op. ---- */
+int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out,
+                  void *stream);
+
+/* ---- R8 combine: out[t] = sum_s scores[t,s] * y[row(t,s)] with
+ * row = inv_perm[t*k+s], or t*k+s when inv_perm is NULL (mlx_take + mlx_multiply +
+ * mlx_sum_axis; mlx-rs/src/ops/reduction.rs:260-276).  y: bf16 [P, H]. ---- */
+int mi_moe_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
+                   int64_t T, int32_t top_k, int32_t hidden, uint16_t *out, void *stream);
+
+/* ---- W: MLX-affine quantize / dequantize of a [rows, cols] fp32 matrix on the
+ * device (mlx_quantize / mlx_dequantize, mlx-rs/src/ops/quantization.rs:50-83,
+ * 124-158).  q: [rows, cols*bits/32]; scales, biases: bf16 [rows, cols/group_size]. */
+int mi_moe_quantize(const float *w, int64_t rows, int64_t cols, int32_t group_size,
+                    int32_t bits, uint32_t *q, uint16_t *scales, uint16_t *biases,
+                    void *stream);
+int mi_moe_dequantize(const uint32_t *q, const uint16_t *scales, const uint16_t *biases,
+                      int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
+                      float *w_hat, void *stream);
+
+/* library version string, e.g. "mi_moe 0.1 gfx950" */
+const char *mi_moe_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_MOE_H */

@@ -1,0 +1,110 @@
+"""ctypes binding of include/mi_moe.h (one function per exported symbol)."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libmi_moe.so")
+
+SCORE_SOFTMAX_THEN_TOPK_RENORM = 0
+SCORE_SOFTMAX_THEN_TOPK = 1
+SCORE_TOPK_THEN_SOFTMAX = 2
+
+# every symbol include/mi_moe.h declares
+EXPORTS = (
+    "mi_moe_last_error", "mi_moe_set_error_handler", "mi_moe_version", "mi_moe_create",
+    "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_route_workspace_size",
+    "mi_moe_route", "mi_moe_dispatch_workspace_size", "mi_moe_dispatch",
+    "mi_moe_gather_qmm_workspace_size", "mi_moe_gather_qmm", "mi_moe_swiglu", "mi_moe_combine",
+    "mi_moe_quantize", "mi_moe_dequantize",
+)
+
+
+class MoeError(RuntimeError):
+    """A non-zero status from the library; ``what`` is the library's message
+    (the role of mlx-rs's ``Exception { what }``, mlx-rs/src/error.rs:162-192)."""
+
+    def __init__(self, what):
+        super().__init__(what)
+        self.what = what
+
+
+class Config(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("hidden", "n_experts", "top_k", "intermediate", "bits", "group_size", "score_mode")]
+
+
+class QMat(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p)]
+
+
+class Weights(C.Structure):
+    _fields_ = [("router_w", C.c_void_p), ("router_bias", C.c_void_p),
+                ("gate", QMat), ("up", QMat), ("down", QMat)]
+
+
+class DebugOut(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in
+                ("topk_idx", "topk_w", "counts", "offsets", "perm", "inv_perm")]
+
+
+ERROR_HANDLER = C.CFUNCTYPE(None, C.c_char_p, C.c_void_p)
+ERROR_DTOR = C.CFUNCTYPE(None, C.c_void_p)
+
+_lib = None
+
+
+def library_path():
+    return _SO
+
+
+def load_library():
+    """Load libmi_moe.so built in-tree by ``__graft_entry__.build()`` (or the Makefile in
+    csrc/).  Raises if it is missing: there is no other code path."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        raise MoeError(f"{_SO} is missing: build it with `make -C {_HERE}/csrc` "
+                       "(or __graft_entry__.build()); there is no fallback path")
+    lib = C.CDLL(_SO)
+    vp, i32, i64, sz = C.c_void_p, C.c_int32, C.c_int64, C.c_size_t
+    lib.mi_moe_last_error.restype = C.c_char_p
+    lib.mi_moe_last_error.argtypes = []
+    lib.mi_moe_version.restype = C.c_char_p
+    lib.mi_moe_version.argtypes = []
+    lib.mi_moe_set_error_handler.restype = None
+    lib.mi_moe_set_error_handler.argtypes = [ERROR_HANDLER, vp, ERROR_DTOR]
+    sigs = {
+        "mi_moe_create": [C.POINTER(Config), C.POINTER(Weights), C.POINTER(vp)],
+        "mi_moe_destroy": [vp],
+        "mi_moe_workspace_size": [C.POINTER(Config), i64, C.POINTER(sz)],
+        "mi_moe_forward": [vp, vp, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
+        "mi_moe_route_workspace_size": [i32, i64, C.POINTER(sz)],
+        "mi_moe_route": [vp, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp, vp, sz, vp],
+        "mi_moe_dispatch_workspace_size": [i32, i64, C.POINTER(sz)],
+        "mi_moe_dispatch": [vp, i64, i32, vp, vp, vp, vp, vp, sz, vp],
+        "mi_moe_gather_qmm_workspace_size": [i32, i64, i32, C.POINTER(sz)],
+        "mi_moe_gather_qmm": [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, i32, i32, i32,
+                              i32, vp, vp, sz, vp],
+        "mi_moe_swiglu": [vp, vp, i64, vp, vp],
+        "mi_moe_combine": [vp, vp, vp, i64, i32, i32, vp, vp],
+        "mi_moe_quantize": [vp, i64, i64, i32, i32, vp, vp, vp, vp],
+        "mi_moe_dequantize": [vp, vp, vp, i64, i64, i32, i32, vp, vp],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def last_error():
+    return load_library().mi_moe_last_error().decode()
+
+
+def check(status):
+    """Turn a status into an exception the way mlx-rs's Guarded::try_from_op does
+    (mlx-rs/src/utils/guard.rs:20-49)."""
+    if status != 0:
+        raise MoeError(last_error())

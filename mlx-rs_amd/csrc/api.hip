@@ -1,0 +1,398 @@
+// C ABI of libmi_moe: validation, workspace carving and the launch sequence of the block.
+// Declarations and the reference interfaces they replace: include/mi_moe.h.
+#include "../../include/mi_moe.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "common.hpp"
+
+using namespace mi_moe;
+
+// ------------------------------------------------------------------ errors
+namespace {
+
+thread_local char g_last_error[512] = "";
+void (*g_handler)(const char *, void *) = nullptr;
+void *g_handler_data = nullptr;
+void (*g_handler_dtor)(void *) = nullptr;
+
+int fail(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+int fail(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
+  va_end(ap);
+  if (g_handler) g_handler(g_last_error, g_handler_data);
+  return 1;
+}
+
+int hip_fail(const char *what, hipError_t e) {
+  return fail("%s: %s", what, hipGetErrorString(e));
+}
+
+#define MI_HIP(call)                                   \
+  do {                                                 \
+    hipError_t e_ = (call);                            \
+    if (e_ != hipSuccess) return hip_fail(#call, e_);  \
+  } while (0)
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
+
+int check_config(const mi_moe_config *c) {
+  if (!c) return fail("config is NULL");
+  if (c->bits != 4 && c->bits != 8) return fail("bits must be 4 or 8, got %d", c->bits);
+  if (c->group_size != 64) return fail("group_size must be 64, got %d", c->group_size);
+  if (c->hidden <= 0 || c->hidden % 64) return fail("hidden must be a positive multiple of 64, got %d", c->hidden);
+  if (c->intermediate <= 0 || c->intermediate % 64)
+    return fail("intermediate must be a positive multiple of 64, got %d", c->intermediate);
+  if (c->n_experts < 1 || c->n_experts > 512) return fail("n_experts must be in [1, 512], got %d", c->n_experts);
+  if (c->top_k < 1 || c->top_k > c->n_experts || c->top_k > 32)
+    return fail("top_k must be in [1, min(n_experts, 32)], got %d", c->top_k);
+  if (c->score_mode < 0 || c->score_mode > 2) return fail("unknown score_mode %d", c->score_mode);
+  return 0;
+}
+
+int check_qmat(const mi_moe_qmat &m, const char *name) {
+  if (!m.w || !m.scales || !m.biases) return fail("%s: weight, scales and biases must be non-NULL", name);
+  if (!aligned16(m.w) || !aligned16(m.scales) || !aligned16(m.biases))
+    return fail("%s: pointers must be 16-byte aligned", name);
+  return 0;
+}
+
+// carve consecutive 256-byte aligned regions out of a workspace
+struct Carver {
+  char *base;
+  size_t off = 0;
+  explicit Carver(void *p) : base(static_cast<char *>(p)) {}
+  template <typename T>
+  T *take(size_t n) {
+    T *p = reinterpret_cast<T *>(base + off);
+    off += align_up(n * sizeof(T));
+    return p;
+  }
+};
+
+struct ForwardWs {
+  uint16_t *logits;
+  uint32_t *topk_idx;
+  uint16_t *topk_w;
+  uint32_t *counts, *offsets, *active, *n_active, *perm, *inv_perm, *src_of;
+  void *disp_scratch;
+  uint16_t *hh, *y;
+  size_t bytes;
+};
+
+ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
+  const int64_t P = T * c.top_k;
+  Carver cv(ws);
+  ForwardWs f;
+  f.logits = cv.take<uint16_t>((size_t)T * c.n_experts);
+  f.topk_idx = cv.take<uint32_t>((size_t)P);
+  f.topk_w = cv.take<uint16_t>((size_t)P);
+  f.counts = cv.take<uint32_t>(c.n_experts);
+  f.offsets = cv.take<uint32_t>(c.n_experts + 1);
+  f.active = cv.take<uint32_t>(c.n_experts);
+  f.n_active = cv.take<uint32_t>(1);
+  f.perm = cv.take<uint32_t>((size_t)P);
+  f.inv_perm = cv.take<uint32_t>((size_t)P);
+  f.src_of = cv.take<uint32_t>((size_t)P);
+  f.disp_scratch = cv.take<char>(dispatch_workspace_bytes(c.n_experts, P));
+  f.hh = cv.take<uint16_t>((size_t)P * c.intermediate);
+  f.y = cv.take<uint16_t>((size_t)P * c.hidden);
+  f.bytes = cv.off;
+  return f;
+}
+
+}  // namespace
+
+struct mi_moe_s {
+  mi_moe_config cfg;
+  mi_moe_weights w;
+};
+
+extern "C" {
+
+const char *mi_moe_last_error(void) { return g_last_error; }
+
+void mi_moe_set_error_handler(void (*handler)(const char *, void *), void *data,
+                              void (*dtor)(void *)) {
+  if (g_handler_dtor && g_handler_data) g_handler_dtor(g_handler_data);
+  g_handler = handler;
+  g_handler_data = data;
+  g_handler_dtor = dtor;
+}
+
+const char *mi_moe_version(void) { return "mi_moe 0.1 gfx950"; }
+
+int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_moe_handle *out) {
+  if (!out) return fail("create: out handle is NULL");
+  if (check_config(cfg)) return 1;
+  if (!weights) return fail("create: weights is NULL");
+  if (!weights->router_w || !aligned16(weights->router_w))
+    return fail("create: router_w must be non-NULL and 16-byte aligned");
+  if (check_qmat(weights->gate, "gate") || check_qmat(weights->up, "up") || check_qmat(weights->down, "down"))
+    return 1;
+  mi_moe_s *h = new (std::nothrow) mi_moe_s;
+  if (!h) return fail("create: out of host memory");
+  h->cfg = *cfg;
+  h->w = *weights;
+  *out = h;
+  return 0;
+}
+
+int mi_moe_destroy(mi_moe_handle h) {
+  delete h;
+  return 0;
+}
+
+int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *bytes) {
+  if (!bytes) return fail("workspace_size: bytes is NULL");
+  if (check_config(cfg)) return 1;
+  if (max_tokens < 0) return fail("workspace_size: negative token count");
+  if (max_tokens * cfg->top_k > (int64_t)1 << 30) return fail("workspace_size: too many (token, expert) pairs");
+  *bytes = carve_forward(*cfg, max_tokens, nullptr).bytes + 256;
+  return 0;
+}
+
+int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
+                   size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream) {
+  if (!h) return fail("forward: handle is NULL");
+  if (T < 0) return fail("forward: negative token count");
+  if (T == 0) return 0;
+  if (!x || !out) return fail("forward: x and out must be non-NULL");
+  if (!aligned16(x) || !aligned16(out)) return fail("forward: x and out must be 16-byte aligned");
+  const mi_moe_config &c = h->cfg;
+  const int64_t P = T * c.top_k;
+  if (P > (int64_t)1 << 30) return fail("forward: too many (token, expert) pairs");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return fail("forward: workspace must be non-NULL and 256-byte aligned");
+  const ForwardWs f = carve_forward(c, T, workspace);
+  if (workspace_bytes < f.bytes)
+    return fail("forward: workspace too small (%zu bytes, need %zu)", workspace_bytes, f.bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+
+  MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st));
+  MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
+  MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
+                         f.src_of, f.active, f.n_active, f.disp_scratch, st));
+  const int max_active = (int)(P < c.n_experts ? P : c.n_experts);
+  GroupedArgs a{};
+  a.row_offsets = f.offsets;
+  a.active = f.active;
+  a.n_active = f.n_active;
+  a.max_active = max_active;
+  a.bits = c.bits;
+  a.total_rows = P;
+  // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
+  a.x = x;
+  a.src_rows = f.src_of;
+  a.dst_rows = nullptr;
+  a.w0 = h->w.gate.w; a.s0 = h->w.gate.scales; a.b0 = h->w.gate.biases;
+  a.w1 = h->w.up.w;   a.s1 = h->w.up.scales;   a.b1 = h->w.up.biases;
+  a.y = f.hh;
+  a.N = c.intermediate;
+  a.K = c.hidden;
+  MI_HIP(launch_grouped_qmm(a, true, st));
+  // down: rows read in sorted order, written back in (token, slot) order
+  a.x = f.hh;
+  a.src_rows = nullptr;
+  a.dst_rows = f.perm;
+  a.w0 = h->w.down.w; a.s0 = h->w.down.scales; a.b0 = h->w.down.biases;
+  a.w1 = nullptr; a.s1 = a.b1 = nullptr;
+  a.y = f.y;
+  a.N = c.hidden;
+  a.K = c.intermediate;
+  MI_HIP(launch_grouped_qmm(a, false, st));
+  MI_HIP(launch_combine(f.y, f.topk_w, nullptr, T, c.top_k, c.hidden, out, st));
+
+  if (dbg) {
+    if (dbg->topk_idx) MI_HIP(hipMemcpyAsync(dbg->topk_idx, f.topk_idx, P * 4, hipMemcpyDeviceToDevice, st));
+    if (dbg->topk_w) MI_HIP(hipMemcpyAsync(dbg->topk_w, f.topk_w, P * 2, hipMemcpyDeviceToDevice, st));
+    if (dbg->counts) MI_HIP(hipMemcpyAsync(dbg->counts, f.counts, c.n_experts * 4, hipMemcpyDeviceToDevice, st));
+    if (dbg->offsets) MI_HIP(hipMemcpyAsync(dbg->offsets, f.offsets, (c.n_experts + 1) * 4, hipMemcpyDeviceToDevice, st));
+    if (dbg->perm) MI_HIP(hipMemcpyAsync(dbg->perm, f.perm, P * 4, hipMemcpyDeviceToDevice, st));
+    if (dbg->inv_perm) MI_HIP(hipMemcpyAsync(dbg->inv_perm, f.inv_perm, P * 4, hipMemcpyDeviceToDevice, st));
+  }
+  return 0;
+}
+
+// ------------------------------------------------------------------ stage level
+
+int mi_moe_route_workspace_size(int32_t n_experts, int64_t T, size_t *bytes) {
+  if (!bytes) return fail("route_workspace_size: bytes is NULL");
+  if (n_experts < 1 || n_experts > 512 || T < 0) return fail("route_workspace_size: bad arguments");
+  *bytes = align_up((size_t)T * n_experts * 2) + 256;
+  return 0;
+}
+
+int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *router_bias, int64_t T,
+                 int32_t hidden, int32_t n_experts, int32_t top_k, int32_t score_mode,
+                 uint32_t *topk_idx, uint16_t *topk_w, uint16_t *logits_out, void *workspace,
+                 size_t workspace_bytes, void *stream) {
+  if (T < 0) return fail("route: negative token count");
+  if (hidden <= 0 || hidden % 64) return fail("route: hidden must be a positive multiple of 64, got %d", hidden);
+  if (n_experts < 1 || n_experts > 512) return fail("route: n_experts must be in [1, 512], got %d", n_experts);
+  if (top_k < 1 || top_k > n_experts || top_k > 32)
+    return fail("route: top_k must be in [1, min(n_experts, 32)], got %d", top_k);
+  if (score_mode < 0 || score_mode > 2) return fail("route: unknown score_mode %d", score_mode);
+  if (T == 0) return 0;
+  if (!x || !router_w || !topk_idx || !topk_w) return fail("route: x, router_w, topk_idx and topk_w must be non-NULL");
+  if (!aligned16(x) || !aligned16(router_w)) return fail("route: x and router_w must be 16-byte aligned");
+  uint16_t *logits = logits_out;
+  if (!logits) {
+    if (!workspace || workspace_bytes < (size_t)T * n_experts * 2)
+      return fail("route: workspace too small (need %zu bytes)", (size_t)T * n_experts * 2);
+    logits = static_cast<uint16_t *>(workspace);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MI_HIP(launch_router_logits(x, router_w, router_bias, T, hidden, n_experts, logits, st));
+  MI_HIP(launch_router_select(logits, T, n_experts, top_k, score_mode, topk_idx, topk_w, st));
+  return 0;
+}
+
+int mi_moe_dispatch_workspace_size(int32_t n_experts, int64_t P, size_t *bytes) {
+  if (!bytes) return fail("dispatch_workspace_size: bytes is NULL");
+  if (n_experts < 1 || n_experts > 512 || P < 0) return fail("dispatch_workspace_size: bad arguments");
+  // scratch + counts/offsets/active/n_active stand-ins for outputs the caller leaves NULL
+  *bytes = align_up(dispatch_workspace_bytes(n_experts, P)) + 4 * align_up((size_t)(n_experts + 1) * 4) + 256;
+  return 0;
+}
+
+int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts, uint32_t *counts,
+                    uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm, void *workspace,
+                    size_t workspace_bytes, void *stream) {
+  if (P < 0 || P > (int64_t)1 << 30) return fail("dispatch: pair count out of range");
+  if (n_experts < 1 || n_experts > 512) return fail("dispatch: n_experts must be in [1, 512], got %d", n_experts);
+  if (!perm) return fail("dispatch: perm must be non-NULL");
+  if (P > 0 && !expert_of_pair) return fail("dispatch: expert_of_pair is NULL");
+  size_t need = 0;
+  mi_moe_dispatch_workspace_size(n_experts, P, &need);
+  if (!workspace || workspace_bytes < need) return fail("dispatch: workspace too small (need %zu bytes)", need);
+  Carver cv(workspace);
+  void *scratch = cv.take<char>(dispatch_workspace_bytes(n_experts, P));
+  uint32_t *active = cv.take<uint32_t>(n_experts + 1);
+  uint32_t *n_active = cv.take<uint32_t>(n_experts + 1);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MI_HIP(launch_dispatch(expert_of_pair, P, n_experts, 1, counts, offsets, perm, inv_perm, nullptr, active,
+                         n_active, scratch, st));
+  return 0;
+}
+
+int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M, size_t *bytes) {
+  if (!bytes) return fail("gather_qmm_workspace_size: bytes is NULL");
+  if (n_experts < 1 || n_experts > 512 || n_idx < 0 || M < 1) return fail("gather_qmm_workspace_size: bad arguments");
+  const int64_t rows = n_idx * M;  // perm and the (src, dst) row maps hold one entry per output row
+  *bytes = align_up(dispatch_workspace_bytes(n_experts, rows)) + 5 * align_up((size_t)(n_experts + 1) * 4) +
+           3 * align_up((size_t)rows * 4) + 256;
+  return 0;
+}
+
+int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                      const uint16_t *biases, const uint32_t *lhs_indices, const uint32_t *rhs_indices,
+                      int64_t n_idx, int64_t x_batch, int32_t M, int32_t N, int32_t K, int32_t n_experts,
+                      int32_t transpose, int32_t group_size, int32_t bits, int32_t sorted_indices,
+                      uint16_t *y, void *workspace, size_t workspace_bytes, void *stream) {
+  (void)sorted_indices;  // a hint in MLX; the segments are rebuilt here either way
+  (void)x_batch;
+  if (!transpose) return fail("gather_qmm: transpose = false is not supported (weights must be [E, N, K*bits/32])");
+  if (bits != 4 && bits != 8) return fail("gather_qmm: bits must be 4 or 8, got %d", bits);
+  if (group_size != 64) return fail("gather_qmm: group_size must be 64, got %d", group_size);
+  if (K <= 0 || K % 64) return fail("gather_qmm: K must be a positive multiple of 64, got %d", K);
+  if (N <= 0 || N % 16) return fail("gather_qmm: N must be a positive multiple of 16, got %d", N);
+  if (M < 1) return fail("gather_qmm: M must be positive, got %d", M);
+  if (n_experts < 1 || n_experts > 512) return fail("gather_qmm: n_experts must be in [1, 512], got %d", n_experts);
+  if (n_idx < 0 || n_idx * M > (int64_t)1 << 30) return fail("gather_qmm: index count out of range");
+  if (n_idx == 0) return 0;
+  if (!x || !w || !scales || !biases || !y) return fail("gather_qmm: x, w, scales, biases and y must be non-NULL");
+  if (!rhs_indices) return fail("gather_qmm: rhs_indices is required");
+  if (!aligned16(x) || !aligned16(w) || !aligned16(scales) || !aligned16(biases) || !aligned16(y))
+    return fail("gather_qmm: pointers must be 16-byte aligned");
+  const int64_t rows = n_idx * M;
+  size_t need = 0;
+  mi_moe_gather_qmm_workspace_size(n_experts, n_idx, M, &need);
+  if (!workspace || workspace_bytes < need) return fail("gather_qmm: workspace too small (need %zu bytes)", need);
+  Carver cv(workspace);
+  void *scratch = cv.take<char>(dispatch_workspace_bytes(n_experts, rows));
+  uint32_t *counts = cv.take<uint32_t>(n_experts + 1);
+  uint32_t *offsets = cv.take<uint32_t>(n_experts + 1);
+  uint32_t *row_offsets = cv.take<uint32_t>(n_experts + 1);
+  uint32_t *active = cv.take<uint32_t>(n_experts + 1);
+  uint32_t *n_active = cv.take<uint32_t>(n_experts + 1);
+  uint32_t *perm = cv.take<uint32_t>((size_t)rows);
+  uint32_t *src_rows = cv.take<uint32_t>((size_t)rows);
+  uint32_t *dst_rows = cv.take<uint32_t>((size_t)rows);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MI_HIP(launch_dispatch(rhs_indices, n_idx, n_experts, 1, counts, offsets, perm, nullptr, nullptr, active,
+                         n_active, scratch, st));
+  MI_HIP(launch_row_maps(perm, lhs_indices, offsets, n_idx, M, n_experts, src_rows, dst_rows, row_offsets, st));
+  GroupedArgs a{};
+  a.x = x;
+  a.src_rows = src_rows;
+  a.dst_rows = dst_rows;
+  a.row_offsets = row_offsets;
+  a.active = active;
+  a.n_active = n_active;
+  a.max_active = (int)(n_idx < n_experts ? n_idx : n_experts);
+  a.w0 = w; a.s0 = scales; a.b0 = biases;
+  a.y = y;
+  a.N = N;
+  a.K = K;
+  a.bits = bits;
+  a.total_rows = rows;
+  MI_HIP(launch_grouped_qmm(a, false, st));
+  return 0;
+}
+
+int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out, void *stream) {
+  if (n < 0) return fail("swiglu: negative element count");
+  if (n == 0) return 0;
+  if (!gate || !up || !out) return fail("swiglu: gate, up and out must be non-NULL");
+  MI_HIP(launch_swiglu(gate, up, n, out, static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+int mi_moe_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm, int64_t T,
+                   int32_t top_k, int32_t hidden, uint16_t *out, void *stream) {
+  if (T < 0) return fail("combine: negative token count");
+  if (top_k < 1) return fail("combine: top_k must be positive, got %d", top_k);
+  if (hidden <= 0 || hidden % 8) return fail("combine: hidden must be a positive multiple of 8, got %d", hidden);
+  if (T == 0) return 0;
+  if (!y || !scores || !out) return fail("combine: y, scores and out must be non-NULL");
+  if (!aligned16(y) || !aligned16(out)) return fail("combine: y and out must be 16-byte aligned");
+  MI_HIP(launch_combine(y, scores, inv_perm, T, top_k, hidden, out, static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+static int check_quant_args(const char *who, int64_t rows, int64_t cols, int32_t group_size, int32_t bits) {
+  if (bits != 2 && bits != 4 && bits != 8) return fail("%s: bits must be 2, 4 or 8, got %d", who, bits);
+  if (group_size != 32 && group_size != 64 && group_size != 128)
+    return fail("%s: group_size must be 32, 64 or 128, got %d", who, group_size);
+  if (rows < 0 || cols < 0) return fail("%s: negative shape", who);
+  if (cols % group_size) return fail("%s: columns (%lld) must be divisible by group_size (%d)", who, (long long)cols, group_size);
+  return 0;
+}
+
+int mi_moe_quantize(const float *w, int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
+                    uint32_t *q, uint16_t *scales, uint16_t *biases, void *stream) {
+  if (check_quant_args("quantize", rows, cols, group_size, bits)) return 1;
+  if (rows * cols == 0) return 0;
+  if (!w || !q || !scales || !biases) return fail("quantize: w, q, scales and biases must be non-NULL");
+  MI_HIP(launch_quantize(w, rows, cols, group_size, bits, q, scales, biases, static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+int mi_moe_dequantize(const uint32_t *q, const uint16_t *scales, const uint16_t *biases, int64_t rows,
+                      int64_t cols, int32_t group_size, int32_t bits, float *w_hat, void *stream) {
+  if (check_quant_args("dequantize", rows, cols, group_size, bits)) return 1;
+  if (rows * cols == 0) return 0;
+  if (!q || !scales || !biases || !w_hat) return fail("dequantize: q, scales, biases and w_hat must be non-NULL");
+  MI_HIP(launch_dequantize(q, scales, biases, rows, cols, group_size, bits, w_hat, static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,118 @@
+// Shared device helpers and internal launcher declarations of libmi_moe (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi_moe {
+
+constexpr int kWave = 64;
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+// ---------------------------------------------------------------- bfloat16
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  return __uint_as_float((uint32_t)h << 16);
+}
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t w) {
+  return __uint_as_float(w & 0xffff0000u);
+}
+// round to nearest even; NaN stays NaN (quiet)
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+// ---------------------------------------------------------------- exp for softmax
+// 2^n * e^r with n = rint(x*log2 e), r by two-step Cody-Waite reduction and a degree-7
+// polynomial, written with explicit fmaf so that no contraction choice of the compiler
+// can change a bit.  Arguments below -80 give 0.  Same formula as the host-side checker.
+__device__ __forceinline__ float det_expf(float x) {
+  if (!(x >= -80.0f)) return 0.0f;
+  if (x > 80.0f) x = 80.0f;
+  float n = __builtin_rintf(x * 1.44269504088896341f);
+  float r = __builtin_fmaf(n, -0.693145751953125f, x);
+  r = __builtin_fmaf(n, -1.42860682030941723e-6f, r);
+  float p = 1.9875691500e-4f;
+  p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+  p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+  p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+  p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+  p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+  float r2 = r * r;
+  float e = __builtin_fmaf(p, r2, r);
+  e = e + 1.0f;
+  int ni = (int)n;
+  float s = __uint_as_float((uint32_t)(ni + 127) << 23);
+  return e * s;
+}
+
+// ---------------------------------------------------------------- wave helpers
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+__device__ __forceinline__ double shfl_xor_f64(double v, int m) {
+  int lo = __double2loint(v), hi = __double2hiint(v);
+  lo = __shfl_xor(lo, m, kWave);
+  hi = __shfl_xor(hi, m, kWave);
+  return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_f64(v, m);
+  return v;
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
+  return v;
+}
+
+// ---------------------------------------------------------------- launchers (host)
+// Each returns hipSuccess or the launch error.  All pointers are device pointers.
+struct GroupedArgs {
+  const uint16_t *x;        // bf16 rows of length K
+  const uint32_t *src_rows; // x row of sorted row r, or nullptr = r
+  const uint32_t *dst_rows; // output row of sorted row r, or nullptr = r
+  const uint32_t *row_offsets; // [E+1] first sorted row of each expert
+  const uint32_t *active;      // [n_active] expert ids with at least one row
+  const uint32_t *n_active;    // device scalar
+  int max_active;              // upper bound of *n_active known on the host
+  const uint32_t *w0, *w1;     // packed weights [E,N,K*bits/32]; w1 only for GLU
+  const uint16_t *s0, *b0, *s1, *b1;
+  uint16_t *y;                 // bf16 [rows, N]
+  int N, K, bits;
+  int64_t total_rows;          // host upper bound on rows (for tile selection)
+};
+
+hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,
+                                int64_t T, int H, int E, uint16_t *logits, hipStream_t st);
+hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k, int mode,
+                                uint32_t *topk_idx, uint16_t *topk_w, hipStream_t st);
+size_t dispatch_workspace_bytes(int E, int64_t P);
+hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
+                           uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
+                           uint32_t *src_of, uint32_t *active, uint32_t *n_active,
+                           void *scratch, hipStream_t st);
+hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
+hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
+                           int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
+                           uint32_t *row_offsets, hipStream_t st);
+hipError_t launch_swiglu(const uint16_t *g, const uint16_t *u, int64_t n, uint16_t *out,
+                         hipStream_t st);
+hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
+                          int64_t T, int k, int H, uint16_t *out, hipStream_t st);
+hipError_t launch_quantize(const float *w, int64_t rows, int64_t cols, int group, int bits,
+                           uint32_t *q, uint16_t *s, uint16_t *b, hipStream_t st);
+hipError_t launch_dequantize(const uint32_t *q, const uint16_t *s, const uint16_t *b,
+                             int64_t rows, int64_t cols, int group, int bits, float *out,
+                             hipStream_t st);
+
+}  // namespace mi_moe

@@ -1,0 +1,255 @@
+// Dispatch: stable sort of the (token, slot) pairs by expert id.
+//
+// Replaces mlx-lm's gather-sort (argsort of the flattened expert indices, argsort of
+// that order, floor_divide by k; mlx-rs/src/ops/sort.rs:75-109,
+// ops/arithmetic.rs:1006-1014, ops/indexing/mod.rs:386-401) with a stable counting
+// sort: per-expert histogram in LDS (ds_add_u32), scans, and a scatter whose ranks are
+// computed from wave ballots in pair order, so the permutation is the one a stable
+// argsort gives, whatever order blocks and waves run in.  Also emits the list of
+// experts that received at least one pair (what the grouped products iterate over).
+#include "common.hpp"
+
+namespace mi_moe {
+
+constexpr int kDispThreads = 1024;             // 16 waves
+constexpr int kDispWaves = kDispThreads / 64;  // pairs per chunk = 1024
+
+__device__ __forceinline__ uint64_t lanemask_lt() {
+  return (1ull << lane_id()) - 1ull;
+}
+
+// lanes (among `valid` ones) that hold the same expert id as this lane
+__device__ __forceinline__ uint64_t match_peers(uint32_t e, int nbits, bool valid) {
+  uint64_t peers = __ballot(valid);
+  for (int b = 0; b < nbits; ++b) {
+    const bool bit = (e >> b) & 1u;
+    const uint64_t bm = __ballot(valid && bit);
+    peers &= bit ? bm : ~bm;
+  }
+  return peers;
+}
+
+// exclusive scan of v[0..n) in LDS by one block of kDispThreads threads (n <= 1024);
+// tmp: n words.  Returns with v holding the exclusive scan and *total the sum.
+__device__ void block_exclusive_scan(uint32_t *v, uint32_t *tmp, int n, uint32_t *total) {
+  const int tid = threadIdx.x;
+  uint32_t mine = tid < n ? v[tid] : 0u;
+  uint32_t *src = v, *dst = tmp;
+  for (int off = 1; off < n; off <<= 1) {
+    uint32_t val = 0;
+    if (tid < n) val = src[tid] + (tid >= off ? src[tid - off] : 0u);
+    __syncthreads();
+    if (tid < n) dst[tid] = val;
+    __syncthreads();
+    uint32_t *t = src;
+    src = dst;
+    dst = t;
+  }
+  uint32_t incl = tid < n ? src[tid] : 0u;
+  __syncthreads();
+  if (tid < n) v[tid] = incl - mine;
+  if (tid == n - 1) *total = incl;
+  __syncthreads();
+}
+
+// Scatter the pairs [j0, j1) (j0 a multiple of 1024) given cur[e] = first free sorted
+// position of expert e for this range.  LDS: cur[E], wcnt[16*E].
+__device__ void scatter_range(const uint32_t *__restrict__ flat, int64_t j0, int64_t j1, int E,
+                              int nbits, int k_div, uint32_t *cur, uint32_t *wcnt,
+                              uint32_t *__restrict__ perm, uint32_t *__restrict__ inv_perm,
+                              uint32_t *__restrict__ src_of) {
+  const int tid = threadIdx.x, wave = tid >> 6;
+  for (int64_t c0 = j0; c0 < j1; c0 += kDispThreads) {
+    for (int i = tid; i < kDispWaves * E; i += kDispThreads) wcnt[i] = 0u;
+    __syncthreads();
+    const int64_t j = c0 + tid;
+    const bool valid = j < j1;
+    uint32_t e = valid ? flat[j] : 0u;
+    e = e < (uint32_t)E ? e : (uint32_t)E - 1u;  // out-of-range ids are clamped, never written past LDS
+    const uint64_t peers = match_peers(e, nbits, valid);
+    const uint32_t rank = __popcll(peers & lanemask_lt());
+    if (valid && rank == 0) wcnt[wave * E + e] = __popcll(peers);
+    __syncthreads();
+    for (int x = tid; x < E; x += kDispThreads) {
+      uint32_t run = cur[x];
+      for (int w = 0; w < kDispWaves; ++w) {
+        uint32_t c = wcnt[w * E + x];
+        wcnt[w * E + x] = run;
+        run += c;
+      }
+      cur[x] = run;
+    }
+    __syncthreads();
+    if (valid) {
+      const uint32_t pos = wcnt[wave * E + e] + rank;
+      perm[pos] = (uint32_t)j;
+      if (inv_perm) inv_perm[j] = pos;
+      if (src_of) src_of[pos] = (uint32_t)j / (uint32_t)k_div;
+    }
+    __syncthreads();
+  }
+}
+
+// counts -> offsets, active list; runs in one block.  LDS cnt[E] in, cur[E] out.
+__device__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E,
+                              uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
+                              uint32_t *__restrict__ active, uint32_t *__restrict__ n_active) {
+  __shared__ uint32_t total;
+  const int tid = threadIdx.x;
+  if (tid < E && counts) counts[tid] = cnt[tid];
+  // active experts in ascending order, by wave 0
+  if (tid < kWave) {
+    uint32_t base = 0;
+    for (int e0 = 0; e0 < E; e0 += kWave) {
+      const int e = e0 + tid;
+      const bool on = e < E && cnt[e] != 0u;
+      const uint64_t bm = __ballot(on);
+      if (on && active) active[base + __popcll(bm & lanemask_lt())] = (uint32_t)e;
+      base += __popcll(bm);
+    }
+    if (tid == 0 && n_active) *n_active = base;
+  }
+  __syncthreads();
+  block_exclusive_scan(cnt, tmp, E, &total);
+  if (tid < E) {
+    cur[tid] = cnt[tid];
+    if (offsets) offsets[tid] = cnt[tid];
+  }
+  if (tid == 0 && offsets) offsets[E] = total;
+  __syncthreads();
+}
+
+// ---- one block does everything (decode-sized P)
+__global__ __launch_bounds__(kDispThreads) void dispatch_single_kernel(
+    const uint32_t *__restrict__ flat, int64_t P, int E, int nbits, int k_div,
+    uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets, uint32_t *__restrict__ perm,
+    uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of,
+    uint32_t *__restrict__ active, uint32_t *__restrict__ n_active) {
+  extern __shared__ uint32_t lds[];
+  uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *wcnt = lds + 3 * E;
+  const int tid = threadIdx.x;
+  for (int i = tid; i < E; i += kDispThreads) cnt[i] = 0u;
+  __syncthreads();
+  for (int64_t j = tid; j < P; j += kDispThreads) {
+    const uint32_t e = flat[j];
+    atomicAdd(&cnt[e < (uint32_t)E ? e : (uint32_t)E - 1u], 1u);
+  }
+  __syncthreads();
+  finish_counts(cnt, tmp, cur, E, counts, offsets, active, n_active);
+  scatter_range(flat, 0, P, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
+}
+
+// ---- three kernels for prefill-sized P: block b owns pairs [b*span, (b+1)*span)
+__global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(
+    const uint32_t *__restrict__ flat, int64_t P, int E, int64_t span,
+    uint32_t *__restrict__ blockhist) {
+  extern __shared__ uint32_t lds[];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < E; i += kDispThreads) lds[i] = 0u;
+  __syncthreads();
+  const int64_t j0 = (int64_t)blockIdx.x * span;
+  const int64_t j1 = j0 + span < P ? j0 + span : P;
+  for (int64_t j = j0 + tid; j < j1; j += kDispThreads) {
+    const uint32_t e = flat[j];
+    atomicAdd(&lds[e < (uint32_t)E ? e : (uint32_t)E - 1u], 1u);
+  }
+  __syncthreads();
+  for (int i = tid; i < E; i += kDispThreads) blockhist[(int64_t)blockIdx.x * E + i] = lds[i];
+}
+
+__global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
+    uint32_t *__restrict__ blockhist, int nb, int E, uint32_t *__restrict__ counts,
+    uint32_t *__restrict__ offsets, uint32_t *__restrict__ active,
+    uint32_t *__restrict__ n_active) {
+  extern __shared__ uint32_t lds[];
+  uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E;
+  const int tid = threadIdx.x;
+  if (tid < E) {
+    uint32_t run = 0;
+    for (int b = 0; b < nb; ++b) run += blockhist[(int64_t)b * E + tid];
+    cnt[tid] = run;
+  }
+  __syncthreads();
+  finish_counts(cnt, tmp, cur, E, counts, offsets, active, n_active);
+  if (tid < E) {  // blockhist[b][e] <- first sorted position of expert e for block b
+    uint32_t run = cur[tid];
+    for (int b = 0; b < nb; ++b) {
+      uint32_t c = blockhist[(int64_t)b * E + tid];
+      blockhist[(int64_t)b * E + tid] = run;
+      run += c;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
+    const uint32_t *__restrict__ flat, int64_t P, int E, int nbits, int k_div, int64_t span,
+    const uint32_t *__restrict__ blockbase, uint32_t *__restrict__ perm,
+    uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of) {
+  extern __shared__ uint32_t lds[];
+  uint32_t *cur = lds, *wcnt = lds + E;
+  const int tid = threadIdx.x;
+  for (int i = tid; i < E; i += kDispThreads) cur[i] = blockbase[(int64_t)blockIdx.x * E + i];
+  __syncthreads();
+  const int64_t j0 = (int64_t)blockIdx.x * span;
+  const int64_t j1 = j0 + span < P ? j0 + span : P;
+  scatter_range(flat, j0, j1, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
+}
+
+constexpr int64_t kSingleMaxP = 4096;
+constexpr int64_t kSpan = 2048;  // pairs per block in the multi-block path
+
+size_t dispatch_workspace_bytes(int E, int64_t P) {
+  if (P <= kSingleMaxP) return 256;
+  int64_t nb = (P + kSpan - 1) / kSpan;
+  return (size_t)nb * E * sizeof(uint32_t) + 256;
+}
+
+hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
+                           uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
+                           uint32_t *src_of, uint32_t *active, uint32_t *n_active,
+                           void *scratch, hipStream_t st) {
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  if (k_div < 1) k_div = 1;
+  if (P <= kSingleMaxP) {
+    size_t lds = (size_t)(3 + kDispWaves) * E * sizeof(uint32_t);
+    dispatch_single_kernel<<<1, kDispThreads, lds, st>>>(flat, P, E, nbits, k_div, counts, offsets,
+                                                        perm, inv_perm, src_of, active, n_active);
+    return hipGetLastError();
+  }
+  uint32_t *blockhist = reinterpret_cast<uint32_t *>(scratch);
+  const int nb = (int)((P + kSpan - 1) / kSpan);
+  dispatch_hist_kernel<<<nb, kDispThreads, (size_t)E * 4, st>>>(flat, P, E, kSpan, blockhist);
+  dispatch_scan_kernel<<<1, kDispThreads, (size_t)3 * E * 4, st>>>(blockhist, nb, E, counts,
+                                                                  offsets, active, n_active);
+  dispatch_scatter_kernel<<<nb, kDispThreads, (size_t)(1 + kDispWaves) * E * 4, st>>>(
+      flat, P, E, nbits, k_div, kSpan, blockhist, perm, inv_perm, src_of);
+  return hipGetLastError();
+}
+
+// Row maps for the stand-alone gather_qmm: sorted position q of index j = perm[q]
+// covers M rows; x rows come from lhs[j]*M + m, outputs go to j*M + m.
+__global__ void row_maps_kernel(const uint32_t *__restrict__ perm, const uint32_t *__restrict__ lhs,
+                                const uint32_t *__restrict__ offsets, int64_t n_idx, int M, int E,
+                                uint32_t *__restrict__ src_rows, uint32_t *__restrict__ dst_rows,
+                                uint32_t *__restrict__ row_offsets) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i <= E) row_offsets[i] = offsets[i] * (uint32_t)M;
+  if (i >= n_idx * M) return;
+  const int64_t q = i / M;
+  const int m = (int)(i % M);
+  const uint32_t j = perm[q];
+  src_rows[i] = (lhs ? lhs[j] : j) * (uint32_t)M + m;
+  dst_rows[i] = j * (uint32_t)M + m;
+}
+
+hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
+                           int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
+                           uint32_t *row_offsets, hipStream_t st) {
+  int64_t n = n_idx * M > E + 1 ? n_idx * M : E + 1;
+  row_maps_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(perm, lhs, offsets, n_idx, M, E,
+                                                              src_rows, dst_rows, row_offsets);
+  return hipGetLastError();
+}
+
+}  // namespace mi_moe

@@ -1,0 +1,224 @@
+// Router: gate Linear -> softmax(precise) -> top-k -> scores.
+//
+// Replaces, for one MoE layer, the MLX primitives a Module would call through
+// mlx-rs: ops::matmul via nn::Linear (mlx-rs/src/nn/linear.rs:84-96,
+// ops/arithmetic.rs:577-603), ops::softmax_axis(precise) (ops/arithmetic.rs:1291-1327),
+// ops::argpartition_axis + slice (ops/sort.rs:211-260), take_along_axis
+// (ops/indexing/mod.rs:433-453), sum_axis + divide (ops/reduction.rs:260-276).
+//
+// Selection must be reproducible bit for bit, so every value the selection depends on
+// is computed in a way that does not depend on summation order:
+//   logits  - fp64 accumulation of exact bf16*bf16 products, rounded fp64->fp32->bf16;
+//   softmax - det_expf terms, fp64 sum, one IEEE fp32 division, rounded to bf16;
+//   top-k   - total order (value descending, expert id ascending), slot 0 = best.
+#include "common.hpp"
+
+namespace mi_moe {
+
+// ------------------------------------------------------------------ logits
+// One wave computes a TM x EM tile of logits: lanes split H in 16-byte pieces, fp64
+// fused multiply-adds, then a butterfly sum.  A block is 4 waves side by side along E.
+template <int TM, int EM>
+__global__ __launch_bounds__(256) void router_logits_kernel(
+    const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg,
+    const float *__restrict__ bias, int64_t T, int H, int E, uint16_t *__restrict__ logits) {
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int64_t t0 = (int64_t)blockIdx.x * TM;
+  const int e0 = (blockIdx.y * 4 + wave) * EM;
+  if (e0 >= E) return;
+
+  const uint16_t *xr[TM];
+  const uint16_t *wr[EM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int64_t t = t0 + i < T ? t0 + i : T - 1;
+    xr[i] = x + t * H;
+  }
+#pragma unroll
+  for (int j = 0; j < EM; ++j) {
+    int e = e0 + j < E ? e0 + j : E - 1;
+    wr[j] = wg + (int64_t)e * H;
+  }
+  double acc[TM][EM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < EM; ++j) acc[i][j] = 0.0;
+
+  for (int h = lane * 8; h < H; h += kWave * 8) {
+    double xd[TM][8], wd[EM][8];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      uint4 v = *reinterpret_cast<const uint4 *>(xr[i] + h);
+      uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        xd[i][2 * q] = (double)bf16lo_to_f32(u[q]);
+        xd[i][2 * q + 1] = (double)bf16hi_to_f32(u[q]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < EM; ++j) {
+      uint4 v = *reinterpret_cast<const uint4 *>(wr[j] + h);
+      uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        wd[j][2 * q] = (double)bf16lo_to_f32(u[q]);
+        wd[j][2 * q + 1] = (double)bf16hi_to_f32(u[q]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < EM; ++j)
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[i][j] = __builtin_fma(xd[i][q], wd[j][q], acc[i][j]);
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < EM; ++j) {
+      double s = wave_sum_f64(acc[i][j]);
+      if (lane == 0 && t0 + i < T && e0 + j < E) {
+        if (bias) s += (double)bias[e0 + j];
+        logits[(t0 + i) * E + e0 + j] = f32_to_bf16((float)s);
+      }
+    }
+}
+
+hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,
+                                int64_t T, int H, int E, uint16_t *logits, hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  if (T <= 64) {
+    dim3 grid((unsigned)T, (unsigned)((E + 3) / 4));
+    router_logits_kernel<1, 1><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+  } else {
+    dim3 grid((unsigned)((T + 3) / 4), (unsigned)((E + 15) / 16));
+    router_logits_kernel<4, 4><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+  }
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------ select
+// float -> unsigned key whose unsigned order is the float order; -0 is mapped to +0 so
+// that the two zeros tie (and the lower expert id wins) as they do in a float compare.
+__device__ __forceinline__ uint32_t ordered_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_to_float(uint32_t k) {
+  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+
+// One wave per token.  Lane l holds experts l, l+64, ... (NV of them).
+template <int NV>
+__global__ __launch_bounds__(256) void router_select_kernel(
+    const uint16_t *__restrict__ logits, int64_t T, int E, int k, int mode,
+    uint32_t *__restrict__ topk_idx, uint16_t *__restrict__ topk_w) {
+  const int lane = lane_id();
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const uint16_t *row = logits + t * E;
+
+  float g[NV], v[NV];
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    int e = j * kWave + lane;
+    g[j] = e < E ? bf16_to_f32(row[e]) : -INFINITY;
+    m = fmaxf(m, g[j]);
+  }
+  if (mode != 2) {
+    m = wave_max_f32(m);
+    float ex[NV];
+    double sum = 0.0;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      int e = j * kWave + lane;
+      ex[j] = e < E ? det_expf(g[j] - m) : 0.0f;
+      sum += (double)ex[j];
+    }
+    sum = wave_sum_f64(sum);
+    const float sf = (float)sum;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[j] = bf16_to_f32(f32_to_bf16(ex[j] / sf));
+  } else {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[j] = g[j];
+  }
+
+  // k rounds of wave-wide arg-max over 64-bit keys (value, then lower id)
+  uint32_t taken = 0;
+  uint32_t my_idx = 0;
+  float my_val = 0.0f;
+  for (int s = 0; s < k; ++s) {
+    uint32_t bk = 0, bi = 0;  // best key / inverted id of this lane
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      int e = j * kWave + lane;
+      if (e < E && !((taken >> j) & 1u)) {
+        uint32_t key = ordered_key(v[j]);
+        uint32_t inv = 0xffffffffu - (uint32_t)e;
+        if (key > bk || (key == bk && inv > bi)) {
+          bk = key;
+          bi = inv;
+        }
+      }
+    }
+#pragma unroll
+    for (int msk = 32; msk >= 1; msk >>= 1) {
+      uint32_t ok = __shfl_xor(bk, msk, kWave), oi = __shfl_xor(bi, msk, kWave);
+      if (ok > bk || (ok == bk && oi > bi)) {
+        bk = ok;
+        bi = oi;
+      }
+    }
+    const uint32_t win = 0xffffffffu - bi;
+    if ((int)(win & (kWave - 1)) == lane) taken |= 1u << (win >> 6);
+    if (lane == s) {
+      my_idx = win;
+      my_val = key_to_float(bk);
+    }
+  }
+
+  // scores; lane s holds slot s
+  float score;
+  if (mode == 2) {
+    const float mx = __shfl(my_val, 0, kWave);  // slot 0 is the largest logit
+    const float e_s = lane < k ? det_expf(my_val - mx) : 0.0f;
+    double sum = 0.0;
+    for (int s = 0; s < k; ++s) sum += (double)__shfl(e_s, s, kWave);
+    score = e_s / (float)sum;
+  } else {
+    score = my_val;
+    if (mode == 0) {
+      float sum = 0.0f;
+      for (int s = 0; s < k; ++s) sum += __shfl(my_val, s, kWave);
+      const float denom = bf16_to_f32(f32_to_bf16(sum));
+      score = my_val / denom;
+    }
+  }
+  if (lane < k) {
+    topk_idx[t * k + lane] = my_idx;
+    topk_w[t * k + lane] = f32_to_bf16(score);
+  }
+}
+
+hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k, int mode,
+                                uint32_t *topk_idx, uint16_t *topk_w, hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  dim3 grid((unsigned)((T + 3) / 4));
+#define MI_SEL(NV) \
+  router_select_kernel<NV><<<grid, 256, 0, st>>>(logits, T, E, k, mode, topk_idx, topk_w)
+  if (E <= 64) MI_SEL(1);
+  else if (E <= 128) MI_SEL(2);
+  else if (E <= 256) MI_SEL(4);
+  else MI_SEL(8);  // E <= 512
+#undef MI_SEL
+  return hipGetLastError();
+}
+
+}  // namespace mi_moe

@@ -1,0 +1,154 @@
+"""Operator-level host API on torch tensors, named after the mlx-rs functions whose MLX
+dispatch each one replaces.  torch supplies device memory and the current stream; all
+arithmetic happens in libmi_moe.so.
+
+dtypes: activations/scales/biases ``torch.bfloat16``; packed weights and indices
+``torch.int32`` holding the uint32 bit patterns (torch has no arithmetic on uint32).
+"""
+import ctypes as C
+
+import torch
+
+from . import capi
+from .capi import check, load_library
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t, dtype, name):
+    if t.dtype != dtype:
+        raise capi.MoeError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if not t.is_cuda:
+        raise capi.MoeError(f"{name}: expected a device tensor")
+    if not t.is_contiguous():
+        raise capi.MoeError(f"{name}: expected a contiguous tensor")
+    return t
+
+
+def _workspace(nbytes, device):
+    return torch.empty(int(nbytes) + 256, dtype=torch.uint8, device=device)
+
+
+def quantize(w, group_size=64, bits=4):
+    """ops::quantize (mlx-rs/src/ops/quantization.rs:50-83): returns (w_q, scales, biases)."""
+    lib = load_library()
+    _need(w, torch.float32, "w")
+    rows, cols = w.shape
+    if cols % max(group_size, 1) or group_size not in (32, 64, 128) or bits not in (2, 4, 8):
+        check(lib.mi_moe_quantize(None, rows, cols, group_size, bits, None, None, None, None))
+    q = torch.empty((rows, cols * bits // 32), dtype=torch.int32, device=w.device)
+    s = torch.empty((rows, cols // group_size), dtype=torch.bfloat16, device=w.device)
+    b = torch.empty_like(s)
+    check(lib.mi_moe_quantize(_ptr(w), rows, cols, group_size, bits, _ptr(q), _ptr(s), _ptr(b), _stream()))
+    return q, s, b
+
+
+def dequantize(w_q, scales, biases, group_size=64, bits=4):
+    """ops::dequantize (mlx-rs/src/ops/quantization.rs:124-158), fp32 result."""
+    lib = load_library()
+    _need(w_q, torch.int32, "w_q")
+    rows = w_q.shape[0]
+    cols = w_q.shape[1] * 32 // bits
+    out = torch.empty((rows, cols), dtype=torch.float32, device=w_q.device)
+    check(lib.mi_moe_dequantize(_ptr(w_q), _ptr(_need(scales, torch.bfloat16, "scales")),
+                                _ptr(_need(biases, torch.bfloat16, "biases")), rows, cols, group_size,
+                                bits, _ptr(out), _stream()))
+    return out
+
+
+def gather_qmm(x, w, scales, biases, lhs_indices=None, rhs_indices=None, transpose=True,
+               group_size=64, bits=4, sorted_indices=False):
+    """ops::gather_qmm (mlx-rs/src/ops/quantization.rs:160-230), same argument order and
+    defaults.  x: bf16 [x_batch, M, K]; w: int32 [E, N, K*bits/32]; indices int32 [n_idx];
+    returns bf16 [n_idx, M, N]."""
+    lib = load_library()
+    _need(x, torch.bfloat16, "x")
+    _need(w, torch.int32, "w")
+    if x.dim() != 3 or w.dim() != 3:
+        raise capi.MoeError("gather_qmm: x must be [batch, M, K] and w [E, N, K*bits/32]")
+    xb, M, K = x.shape
+    E, N = w.shape[0], w.shape[1]
+    if rhs_indices is None:
+        raise capi.MoeError("gather_qmm: rhs_indices is required")
+    n_idx = rhs_indices.numel()
+    y = torch.empty((n_idx, M, N), dtype=torch.bfloat16, device=x.device)
+    need = C.c_size_t()
+    check(lib.mi_moe_gather_qmm_workspace_size(E, n_idx, M, C.byref(need)))
+    ws = _workspace(need.value, x.device)
+    check(lib.mi_moe_gather_qmm(
+        _ptr(x), _ptr(w), _ptr(_need(scales, torch.bfloat16, "scales")),
+        _ptr(None if biases is None else _need(biases, torch.bfloat16, "biases")),
+        _ptr(None if lhs_indices is None else _need(lhs_indices, torch.int32, "lhs_indices")),
+        _ptr(_need(rhs_indices, torch.int32, "rhs_indices")), n_idx, xb, M, N, K, E, int(transpose),
+        group_size, bits, int(sorted_indices), _ptr(y), _ptr(ws), ws.numel(), _stream()))
+    return y
+
+
+def route(x, router_w, top_k, score_mode=capi.SCORE_SOFTMAX_THEN_TOPK_RENORM, router_bias=None,
+          return_logits=False):
+    """Gate Linear + softmax(precise) + top-k + scores in one call (what an mlx-lm MoE block
+    does with matmul / softmax_axis / argpartition_axis / take_along_axis / sum_axis / divide).
+    Returns (inds int32 [T,k], scores bf16 [T,k][, logits bf16 [T,E]])."""
+    lib = load_library()
+    _need(x, torch.bfloat16, "x")
+    _need(router_w, torch.bfloat16, "router_w")
+    T, H = x.shape
+    E = router_w.shape[0]
+    inds = torch.empty((T, top_k), dtype=torch.int32, device=x.device)
+    sc = torch.empty((T, top_k), dtype=torch.bfloat16, device=x.device)
+    logits = torch.empty((T, E), dtype=torch.bfloat16, device=x.device)
+    check(lib.mi_moe_route(_ptr(x), _ptr(router_w),
+                           _ptr(None if router_bias is None else _need(router_bias, torch.float32, "router_bias")),
+                           T, H, E, top_k, score_mode, _ptr(inds), _ptr(sc), _ptr(logits), None, 0, _stream()))
+    return (inds, sc, logits) if return_logits else (inds, sc)
+
+
+def dispatch(expert_of_pair, n_experts):
+    """Stable sort of the pairs by expert: returns (counts, offsets, perm, inv_perm), the
+    results of mlx-lm's argsort / argsort / floor_divide sequence plus the histogram."""
+    lib = load_library()
+    flat = _need(expert_of_pair, torch.int32, "expert_of_pair").reshape(-1)
+    P = flat.numel()
+    dev = flat.device
+    counts = torch.empty(n_experts, dtype=torch.int32, device=dev)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    perm = torch.empty(P, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    need = C.c_size_t()
+    check(lib.mi_moe_dispatch_workspace_size(n_experts, P, C.byref(need)))
+    ws = _workspace(need.value, dev)
+    check(lib.mi_moe_dispatch(_ptr(flat), P, n_experts, _ptr(counts), _ptr(offsets), _ptr(perm), _ptr(inv),
+                              _ptr(ws), ws.numel(), _stream()))
+    return counts, offsets, perm, inv
+
+
+def swiglu(gate, up):
+    """nn::silu(gate) * up on bf16 tensors (mlx-rs/src/nn/activation.rs:142-144)."""
+    lib = load_library()
+    _need(gate, torch.bfloat16, "gate")
+    _need(up, torch.bfloat16, "up")
+    if gate.shape != up.shape:
+        raise capi.MoeError("swiglu: gate and up must have the same shape")
+    out = torch.empty_like(gate)
+    check(lib.mi_moe_swiglu(_ptr(gate), _ptr(up), gate.numel(), _ptr(out), _stream()))
+    return out
+
+
+def combine(y, scores, inv_perm=None):
+    """(y[inv] * scores[..., None]).sum(-2): y bf16 [P, H], scores bf16 [T, k] -> bf16 [T, H]."""
+    lib = load_library()
+    _need(y, torch.bfloat16, "y")
+    _need(scores, torch.bfloat16, "scores")
+    T, k = scores.shape
+    H = y.shape[-1]
+    out = torch.empty((T, H), dtype=torch.bfloat16, device=y.device)
+    check(lib.mi_moe_combine(_ptr(y), _ptr(scores),
+                             _ptr(None if inv_perm is None else _need(inv_perm, torch.int32, "inv_perm")),
+                             T, k, H, _ptr(out), _stream()))
+    return out

@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized MoE layer on one MI355X.
+
+Default workload = the Qwen3-30B-A3B-shaped layer at decode (hidden 2048, 128 experts,
+top-8 renormalised, intermediate 768, 4-bit g64), batches 1 / 8 / 32; the headline
+`value` is tokens/s at batch 32.  A "step" is one forward of the layer over one batch
+whose inputs are already in HBM.  Steps rotate over several distinct weight sets whose
+total size exceeds the 256 MB Infinity Cache, so weights stream from HBM every step.
+
+Prints ONE JSON line (see --help for the other workloads).  The CPU-baseline leg times
+the CPU oracle (a restatement of the MLX CPU op sequence; MLX itself is not available)
+on the host cores; it is the only part of this script that touches oracle/.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="decode",
+                    choices=["decode", "prefill", "mixtral_decode", "mixtral_prefill", "qwen3_235b_prefill", "tiny"])
+    ap.add_argument("--layers", type=int, default=0, help="distinct weight sets to rotate over (0 = auto)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args()
+
+
+WORKLOADS = {
+    # name: (config key, batches, headline batch, zipf s, bound)
+    "decode": ("qwen3_30b_a3b", [1, 8, 32], 32, None, "hbm"),
+    "prefill": ("qwen3_30b_a3b", [4096], 4096, 1.1, "mfma"),
+    "mixtral_decode": ("mixtral_8x7b", [1], 1, None, "hbm"),
+    "mixtral_prefill": ("mixtral_8x7b", [2048], 2048, None, "mfma"),
+    "qwen3_235b_prefill": ("qwen3_235b_a22b", [8192], 8192, 1.3, "mfma"),
+    "tiny": ("tiny", [32], 32, None, "hbm"),
+}
+
+
+def time_steps(fn, steps, warmup, torch):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(warmup + i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import mlx_rs_amd as m
+    from mlx_rs_amd import synth
+
+    m.load_library()  # raises if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    cfg_name, batches, headline, zipf_s, bound = WORKLOADS[args.workload]
+    cfg = synth.CONFIGS[cfg_name]
+    per_expert = synth.layer_bytes_per_expert(cfg)
+    layer_bytes = per_expert * cfg.n_experts
+    n_layers = args.layers or max(2, min(8, int(1.4e9 // layer_bytes) + 1))
+    if layer_bytes > 1.0e9:
+        n_layers = args.layers or 2
+    blocks = [synth.make_block(cfg, seed=args.seed + 31 * i, device=dev, zipf_s=zipf_s, gen_device="cuda")
+              for i in range(n_layers)]
+    torch.cuda.synchronize()
+
+    detail = {}
+    head = None
+    for T in batches:
+        x = synth.make_tokens(cfg, T, seed=args.seed, device=dev)
+        outs = [torch.empty_like(x) for _ in range(n_layers)]
+        for b in blocks:
+            b.reserve(T)
+        # realised routing (per weight set)
+        actives, counts_stats = [], []
+        for b in blocks:
+            _, dbg = b.forward(x, debug=True)
+            c = dbg["counts"].cpu().numpy()
+            actives.append(int((c > 0).sum()))
+            counts_stats.append((int(c.max()), float(c.mean()), int(c.min())))
+        n_active = sum(actives) / len(actives)
+
+        graph = None
+        if not args.no_graph:
+            # one graph replays a forward through every weight set (launch overhead amortised the
+            # way a serving loop would capture a whole decode step)
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                for i, b in enumerate(blocks):
+                    b.forward(x, out=outs[i])
+            torch.cuda.current_stream().wait_stream(s)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i, b in enumerate(blocks):
+                    b.forward(x, out=outs[i])
+            eager_ref = [o.clone() for o in outs]
+            graph.replay()
+            torch.cuda.synchronize()
+            for o, r in zip(outs, eager_ref):
+                assert torch.equal(o, r), "graph replay differs from the eager result"
+
+        if graph is not None:
+            # a step = one forward; one replay = n_layers steps
+            reps = max(1, args.steps // n_layers)
+            wreps = max(1, args.warmup // n_layers)
+            ms = time_steps(lambda i: graph.replay(), reps, wreps, torch) / n_layers
+            steps_done = reps * n_layers
+        else:
+            ms = time_steps(lambda i: blocks[i % n_layers].forward(x, out=outs[i % n_layers]),
+                            args.steps, args.warmup, torch)
+            steps_done = args.steps
+        eager_ms = time_steps(lambda i: blocks[i % n_layers].forward(x, out=outs[i % n_layers]),
+                              args.steps, args.warmup, torch)
+
+        # per-kernel durations from HIP events on the launch stream, same K steps
+        stage = [0.0] * m.capi.N_STAGES
+        for i in range(args.steps):
+            _, st = blocks[i % n_layers].forward_timed(x, out=outs[i % n_layers])
+            stage = [a + b for a, b in zip(stage, st)]
+        stage = [v / args.steps for v in stage]
+
+        P = T * cfg.top_k
+        qbytes = lambda n, k: n * k * cfg.bits // 8 + (n * k // cfg.group_size) * 4
+        gu_bytes = n_active * 2 * qbytes(cfg.intermediate, cfg.hidden) + T * cfg.hidden * 2 + P * cfg.intermediate * 2
+        dn_bytes = n_active * qbytes(cfg.hidden, cfg.intermediate) + P * cfg.intermediate * 2 + P * cfg.hidden * 2
+        alg_bytes = synth.decode_algorithmic_bytes(cfg, T, n_active)
+        flops = synth.prefill_flops(cfg, T)
+        gu_flops = P * 2 * 2 * cfg.hidden * cfg.intermediate
+        detail[str(T)] = {
+            "tokens_per_s": T / (ms * 1e-3), "ms_per_step": ms, "ms_per_step_eager": eager_ms,
+            "steps": steps_done, "active_experts": n_active,
+            "counts_max_mean_min": counts_stats[0],
+            "layer_algorithmic_MB": alg_bytes / 1e6, "layer_GBps": alg_bytes / (ms * 1e-3) / 1e9,
+            "layer_hbm_frac": alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "layer_TFLOPs": flops / (ms * 1e-3) / 1e12,
+            "layer_mfma_frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "stage_us": {n: round(v * 1e3, 2) for n, v in zip(m.capi.STAGE_NAMES, stage)},
+            "gate_up_GBps": gu_bytes / (stage[3] * 1e-3) / 1e9,
+            "down_GBps": dn_bytes / (stage[4] * 1e-3) / 1e9,
+            "gate_up_TFLOPs": gu_flops / (stage[3] * 1e-3) / 1e12,
+        }
+        if T == headline:
+            head = dict(ms=ms, T=T, gu_bytes=gu_bytes, gu_ms=stage[3], gu_flops=gu_flops, steps=steps_done)
+        del outs, graph
+
+    if bound == "hbm":
+        achieved = head["gu_bytes"] / (head["gu_ms"] * 1e-3) / 1e9
+        roofline = {"kernel": "qmm_small_kernel (gate/up + SwiGLU)", "bound": "hbm", "achieved": achieved,
+                    "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None}
+    else:
+        achieved = head["gu_flops"] / (head["gu_ms"] * 1e-3) / 1e12
+        roofline = {"kernel": "grouped qmm (gate/up + SwiGLU)", "bound": "mfma", "achieved": achieved,
+                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                    "traffic": None}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(cfg, blocks[0], headline, args.seed, synth)
+
+    out = {
+        "metric": "MoE-layer tokens/sec (%s)" % ("decode" if bound == "hbm" else "prefill"),
+        "value": headline / (head["ms"] * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": head["steps"], "warmup": args.warmup, "ms_per_step": head["ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "%s %s-bit g64 MoE layer, %s, batch %d" % (cfg_name, cfg.bits, args.workload, headline),
+                   "hidden": cfg.hidden, "n_experts": cfg.n_experts, "top_k": cfg.top_k,
+                   "intermediate": cfg.intermediate, "bits": cfg.bits, "batch": headline,
+                   "weight_sets_rotated": n_layers, "launch": "eager" if args.no_graph else "hip-graph"},
+        "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
+    }
+    print(json.dumps(out))
+
+
+def cpu_baseline(cfg, block, T, seed, synth):
+    """Times the CPU oracle (op-by-op 'strict' mode: the MLX CPU op sequence restated) on the
+    host cores for the same layer and batch; a bounded sample (a few repeats, or a token
+    subsample for the large prefill shapes)."""
+    import numpy as np
+    import oracle
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from helpers import bits_u16, bits_u32
+
+    threads = min(16, len(os.sched_getaffinity(0)))
+    W = dict(router_w=bits_u16(block.gate_weight),
+             router_bias=None if block.router_bias is None else block.router_bias.cpu().numpy(),
+             gate=(bits_u32(block.gate_proj.weight), bits_u16(block.gate_proj.scales), bits_u16(block.gate_proj.biases)),
+             up=(bits_u32(block.up_proj.weight), bits_u16(block.up_proj.scales), bits_u16(block.up_proj.biases)),
+             down=(bits_u32(block.down_proj.weight), bits_u16(block.down_proj.scales), bits_u16(block.down_proj.biases)))
+    Ts = min(T, 256)
+    x = bits_u16(synth.make_tokens(cfg, Ts, seed=seed, device="cpu"))
+    ocfg = oracle.make_config(cfg.hidden, cfg.n_experts, cfg.top_k, cfg.intermediate, cfg.bits, cfg.group_size,
+                              cfg.score_mode)
+    oracle.moe_forward(ocfg, W, x, strict=True, n_threads=threads, debug=False)  # warm-up
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 or (time.perf_counter() - t_all < 10.0 and len(times) < 50):
+        t0 = time.perf_counter()
+        oracle.moe_forward(ocfg, W, x, strict=True, n_threads=threads, debug=False)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    sample = "%d runs of the full layer at batch %d" % (len(times), Ts)
+    if Ts != T:
+        sample += " (token subsample of the %d-token workload; tokens/s is per token, so no scaling applied)" % T
+    return {"value": Ts / med, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": sample + "; CPU oracle in op-by-op mode, OpenMP"}
+
+
+if __name__ == "__main__":
+    main()

@@ -102,6 +102,15 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
                    void *workspace, size_t workspace_bytes, const mi_moe_debug_out *dbg,
                    void *stream);
 
+/* The same forward with a HIP event recorded on `stream` before the first launch and
+ * after each stage; waits for the last one and returns the MI_MOE_N_STAGES elapsed times
+ * in milliseconds (host array): router logits, router select, dispatch, gate/up + SwiGLU,
+ * down, combine.  For measurement; mlx-rs has no counterpart (it times with
+ * Instant::now() around eval, mlx-rs/examples/linear_regression.rs:40-59). */
+#define MI_MOE_N_STAGES 6
+int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
+                         void *workspace, size_t workspace_bytes, void *stream, float *stage_ms);
+
 /* ---- R1-R4 router: gate Linear + softmax(precise) + argpartition top-k +
  * take_along_axis + renormalise (mlx_matmul, mlx_softmax_axis, mlx_argpartition_axis,
  * mlx_take_along_axis, mlx_sum_axis, mlx_divide; mlx-rs/src/ops/arithmetic.rs:577-603,

@@ -8,11 +8,14 @@ _SO = os.path.join(_HERE, "libmi_moe.so")
 SCORE_SOFTMAX_THEN_TOPK_RENORM = 0
 SCORE_SOFTMAX_THEN_TOPK = 1
 SCORE_TOPK_THEN_SOFTMAX = 2
+N_STAGES = 6
+STAGE_NAMES = ("router_logits", "router_select", "dispatch", "gate_up_swiglu", "down", "combine")
 
 # every symbol include/mi_moe.h declares
 EXPORTS = (
     "mi_moe_last_error", "mi_moe_set_error_handler", "mi_moe_version", "mi_moe_create",
-    "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_route_workspace_size",
+    "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_forward_timed",
+    "mi_moe_route_workspace_size",
     "mi_moe_route", "mi_moe_dispatch_workspace_size", "mi_moe_dispatch",
     "mi_moe_gather_qmm_workspace_size", "mi_moe_gather_qmm", "mi_moe_swiglu", "mi_moe_combine",
     "mi_moe_quantize", "mi_moe_dequantize",
@@ -79,6 +82,7 @@ def load_library():
         "mi_moe_destroy": [vp],
         "mi_moe_workspace_size": [C.POINTER(Config), i64, C.POINTER(sz)],
         "mi_moe_forward": [vp, vp, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
+        "mi_moe_forward_timed": [vp, vp, i64, vp, vp, sz, vp, C.POINTER(C.c_float)],
         "mi_moe_route_workspace_size": [i32, i64, C.POINTER(sz)],
         "mi_moe_route": [vp, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp, vp, sz, vp],
         "mi_moe_dispatch_workspace_size": [i32, i64, C.POINTER(sz)],

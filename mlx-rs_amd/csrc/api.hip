@@ -54,6 +54,9 @@ int check_config(const mi_moe_config *c) {
   if (c->top_k < 1 || c->top_k > c->n_experts || c->top_k > 32)
     return fail("top_k must be in [1, min(n_experts, 32)], got %d", c->top_k);
   if (c->score_mode < 0 || c->score_mode > 2) return fail("unknown score_mode %d", c->score_mode);
+  if (c->bits == 4 && (c->hidden % 128 || c->intermediate % 128))
+    return fail("4-bit weights need hidden and intermediate to be multiples of 128 (got %d, %d)", c->hidden,
+                c->intermediate);
   return 0;
 }
 
@@ -159,8 +162,11 @@ int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *
   return 0;
 }
 
-int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
-                   size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream) {
+// The launch sequence of one forward.  ev: nullptr, or kStages + 1 events recorded on the
+// stream before the first launch and after each stage.
+static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
+                        size_t workspace_bytes, const mi_moe_debug_out *dbg, hipStream_t st,
+                        hipEvent_t *ev) {
   if (!h) return fail("forward: handle is NULL");
   if (T < 0) return fail("forward: negative token count");
   if (T == 0) return 0;
@@ -174,12 +180,20 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
   const ForwardWs f = carve_forward(c, T, workspace);
   if (workspace_bytes < f.bytes)
     return fail("forward: workspace too small (%zu bytes, need %zu)", workspace_bytes, f.bytes);
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  int stage = 0;
+#define MI_STAGE_DONE()                                  \
+  do {                                                   \
+    if (ev) MI_HIP(hipEventRecord(ev[++stage], st));     \
+  } while (0)
+  if (ev) MI_HIP(hipEventRecord(ev[0], st));
 
   MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st));
+  MI_STAGE_DONE();
   MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
+  MI_STAGE_DONE();
   MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
                          f.src_of, f.active, f.n_active, f.disp_scratch, st));
+  MI_STAGE_DONE();
   const int max_active = (int)(P < c.n_experts ? P : c.n_experts);
   GroupedArgs a{};
   a.row_offsets = f.offsets;
@@ -188,6 +202,7 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
   a.max_active = max_active;
   a.bits = c.bits;
   a.total_rows = P;
+  a.max_rows_per_expert = T;  // a token picks an expert at most once
   // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
   a.x = x;
   a.src_rows = f.src_of;
@@ -198,6 +213,7 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
   a.N = c.intermediate;
   a.K = c.hidden;
   MI_HIP(launch_grouped_qmm(a, true, st));
+  MI_STAGE_DONE();
   // down: rows read in sorted order, written back in (token, slot) order
   a.x = f.hh;
   a.src_rows = nullptr;
@@ -208,7 +224,10 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
   a.N = c.hidden;
   a.K = c.intermediate;
   MI_HIP(launch_grouped_qmm(a, false, st));
+  MI_STAGE_DONE();
   MI_HIP(launch_combine(f.y, f.topk_w, nullptr, T, c.top_k, c.hidden, out, st));
+  MI_STAGE_DONE();
+#undef MI_STAGE_DONE
 
   if (dbg) {
     if (dbg->topk_idx) MI_HIP(hipMemcpyAsync(dbg->topk_idx, f.topk_idx, P * 4, hipMemcpyDeviceToDevice, st));
@@ -219,6 +238,30 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
     if (dbg->inv_perm) MI_HIP(hipMemcpyAsync(dbg->inv_perm, f.inv_perm, P * 4, hipMemcpyDeviceToDevice, st));
   }
   return 0;
+}
+
+int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
+                   size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream) {
+  return forward_impl(h, x, T, out, workspace, workspace_bytes, dbg, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
+                         size_t workspace_bytes, void *stream, float *stage_ms) {
+  if (!stage_ms) return fail("forward_timed: stage_ms is NULL");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipEvent_t ev[MI_MOE_N_STAGES + 1];
+  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) MI_HIP(hipEventCreate(&ev[i]));
+  int rc = forward_impl(h, x, T, out, workspace, workspace_bytes, nullptr, st, ev);
+  if (rc == 0 && T > 0) {
+    hipError_t e = hipEventSynchronize(ev[MI_MOE_N_STAGES]);
+    if (e != hipSuccess) rc = hip_fail("hipEventSynchronize", e);
+    for (int i = 0; rc == 0 && i < MI_MOE_N_STAGES; ++i) {
+      e = hipEventElapsedTime(&stage_ms[i], ev[i], ev[i + 1]);
+      if (e != hipSuccess) rc = hip_fail("hipEventElapsedTime", e);
+    }
+  }
+  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) hipEventDestroy(ev[i]);
+  return rc;
 }
 
 // ------------------------------------------------------------------ stage level
@@ -303,6 +346,7 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   if (bits != 4 && bits != 8) return fail("gather_qmm: bits must be 4 or 8, got %d", bits);
   if (group_size != 64) return fail("gather_qmm: group_size must be 64, got %d", group_size);
   if (K <= 0 || K % 64) return fail("gather_qmm: K must be a positive multiple of 64, got %d", K);
+  if (bits == 4 && K % 128) return fail("gather_qmm: 4-bit weights need K to be a multiple of 128, got %d", K);
   if (N <= 0 || N % 16) return fail("gather_qmm: N must be a positive multiple of 16, got %d", N);
   if (M < 1) return fail("gather_qmm: M must be positive, got %d", M);
   if (n_experts < 1 || n_experts > 512) return fail("gather_qmm: n_experts must be in [1, 512], got %d", n_experts);
@@ -344,6 +388,7 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   a.K = K;
   a.bits = bits;
   a.total_rows = rows;
+  a.max_rows_per_expert = rows;
   MI_HIP(launch_grouped_qmm(a, false, st));
   return 0;
 }

@@ -20,15 +20,23 @@ __device__ __forceinline__ float bf16lo_to_f32(uint32_t w) { return __uint_as_fl
 __device__ __forceinline__ float bf16hi_to_f32(uint32_t w) {
   return __uint_as_float(w & 0xffff0000u);
 }
-// round to nearest even; NaN stays NaN (quiet)
+// round to nearest even; NaN stays NaN (quiet).  Integer arithmetic only: the bits are the
+// same as the host-side checker's on every input.
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x40u) : r);
 }
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+// two floats -> packed bf16 with the hardware converter (v_cvt_pk_bf16_f32, round to nearest
+// even): for values that only have to be within tolerance
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // ---------------------------------------------------------------- exp for softmax
@@ -90,6 +98,7 @@ struct GroupedArgs {
   uint16_t *y;                 // bf16 [rows, N]
   int N, K, bits;
   int64_t total_rows;          // host upper bound on rows (for tile selection)
+  int64_t max_rows_per_expert; // host upper bound on the longest segment
 };
 
 hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,

@@ -11,6 +11,8 @@
 // group, in fp32.  The integer codes are exact in bf16, so the matrix cores multiply raw
 // codes (no per-element dequantisation, no rounding of w_hat), and scale and bias are
 // applied once per group to the fp32 partial sums.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace mi_moe {
@@ -21,6 +23,17 @@ __device__ __forceinline__ f32x4_t mfma16(const uint32_t (&a)[4], const uint32_t
   u32x4_t av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
                                                  __builtin_bit_cast(bf16x8_t, bv), c, 0, 0, 0);
+}
+
+// (a & mask) | orv.  With mask and orv held in registers (see opaque_reg) this is one
+// v_and_or_b32; as literals it would be two instructions (VOP3 takes no 32-bit literals).
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
+  return (a & mask) | orv;
+}
+// hide a constant from the optimiser so that it stays in a register
+__device__ __forceinline__ uint32_t opaque_reg(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
 }
 
 __device__ __forceinline__ float silu_mul(float g, float u) {
@@ -48,123 +61,238 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
 //
 // KW waves of a block split K chunk-wise (wave wk takes chunks wk, wk+KW, ...), the other
 // 4/KW waves take further row tiles; partial sums meet in LDS and are added in wave order.
-template <int BITS, bool GLU, int KW>
-__global__ __launch_bounds__(256) void qmm_small_kernel(GroupedArgs a) {
-  constexpr int NW = 4 / KW;                    // row tiles per block
-  constexpr int TT = BITS == 4 ? 8 : 16;        // tokens per tile
-  constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one uint4 per lane)
-  constexpr int XV = BITS == 4 ? 4 : 2;         // uint4 of activations per lane per chunk
-  constexpr int NM = GLU ? 2 : 1;
+#ifndef MI_MOE_RING
+#define MI_MOE_RING 4
+#endif
 
-  if (blockIdx.y >= *a.n_active) return;
-  const int e = (int)a.active[blockIdx.y];
-  const int lane = lane_id(), wave = threadIdx.x >> 6;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+
+// Buffer resource over [base, base + bytes): loads past the end return 0, addresses are
+// a wave-uniform descriptor + a 32-bit lane offset + a scalar offset (no 64-bit VGPR math).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+template <int BITS, bool GLU>
+struct ChunkRegs {
+  static constexpr int NM = GLU ? 2 : 1;
+  u32x4_t q[NM];    // packed codes of this lane's weight row
+  uint32_t sc[NM];  // raw bf16 scale of the group this lane's D rows belong to
+};
+
+// LDS layout of one token tile (all offsets 16-byte aligned):
+//   [0, (tt+1)*xstride)            tt staged activation rows + one all-zero row
+//   then 2 x 16 x gpad bf16        per-(token, group) sums of x, split hi / lo, rows >= nt zero
+// xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
+__host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
+__host__ __device__ constexpr int gpad_of(int K) { return (K / 64 + 31) / 32 * 32; }
+__host__ __device__ constexpr int gsum_stride_bytes(int K) { return 2 * gpad_of(K) + 16; }
+__host__ __device__ constexpr size_t small_lds_bytes(int K, int tt) {
+  return (size_t)(tt + 1) * x_stride_bytes(K) + 2 * 16 * (size_t)gsum_stride_bytes(K);
+}
+
+template <int BITS, bool GLU, int KW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8)))
+void qmm_small_kernel(GroupedArgs a, int tt) {
+  constexpr int NW = 4 / KW;                    // row tiles per block
+  constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one 16-byte load per lane)
+  constexpr int XV = BITS == 4 ? 4 : 2;         // 16-byte pieces of activations per lane per chunk
+  constexpr int NM = GLU ? 2 : 1;
+  constexpr int D = MI_MOE_RING;                // chunks kept in flight per wave
+  using Regs = ChunkRegs<BITS, GLU>;
+
+  const uint32_t n_act = *a.n_active;
+  const uint32_t e_raw = a.active[blockIdx.y];  // the list has room for every expert
+  if (blockIdx.y >= n_act) return;
+  const int e = (int)e_raw;
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction
   const int wk = wave % KW, wn = wave / KW;
   const int c = lane & 15, kb = lane >> 4;
   const int N = a.N, K = a.K;
-  const int64_t r0 = a.row_offsets[e];
-  const int cnt = (int)(a.row_offsets[e + 1] - a.row_offsets[e]);
   const int n0 = (blockIdx.x * NW + wn) * 16;
   const bool tile_ok = n0 < N;
-  const int n = tile_ok ? n0 + c : 0;  // weight row of this lane (B operand / D column)
+  const int n = n0 + c;  // weight row of this lane (B operand / D column); rows >= N load zeros
 
-  const int words_per_row = K * BITS / 32;
+  const int row_bytes = K * BITS / 8;
   const int groups_per_row = K / 64;
-  const int nchunks = (K + CH - 1) / CH;
-  const int64_t wrow = ((int64_t)e * N + n);
-  const uint32_t *wp[NM];
-  const uint16_t *sp[NM], *bp[NM];
-  wp[0] = a.w0 + wrow * words_per_row;
-  sp[0] = a.s0 + wrow * groups_per_row;
-  bp[0] = a.b0 + wrow * groups_per_row;
-  if constexpr (GLU) {
-    wp[1] = a.w1 + wrow * words_per_row;
-    sp[1] = a.s1 + wrow * groups_per_row;
-    bp[1] = a.b1 + wrow * groups_per_row;
-  }
-  const uint32_t ones[4] = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  const int nchunks = K / CH;
+  const int cpw = (nchunks + KW - 1) / KW;  // contiguous K range per wave
+  const int ch0 = wk * cpw;
+  const int ch1 = ch0 + cpw < nchunks ? ch0 + cpw : nchunks;
 
+  // one descriptor per tensor of this expert
+  const int64_t ebase = (int64_t)e * N;
+  __amdgpu_buffer_rsrc_t wr[NM], sr[NM], br[NM];
+  wr[0] = make_rsrc(a.w0 + ebase * (row_bytes / 4), (uint32_t)N * row_bytes);
+  sr[0] = make_rsrc(a.s0 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
+  br[0] = make_rsrc(a.b0 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
+  if constexpr (GLU) {
+    wr[1] = make_rsrc(a.w1 + ebase * (row_bytes / 4), (uint32_t)N * row_bytes);
+    sr[1] = make_rsrc(a.s1 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
+    br[1] = make_rsrc(a.b1 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
+  }
+  const uint32_t w_voff = (uint32_t)n * row_bytes + kb * 16;  // lane kb: 16 bytes of the 64-byte chunk
+  const uint32_t g_voff = (uint32_t)n * groups_per_row * 2;
+  // 4-bit: D rows 0-7 (lanes kb < 2) belong to a chunk's first group, rows 8-15 to its second
+  const uint32_t s_voff = g_voff + (BITS == 4 ? (kb >> 1) * 2 : 0);
+
+  // issue every global load of chunk ch into R
+  auto issue = [&](int ch, Regs &R) {
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      R.q[m] = __builtin_amdgcn_raw_buffer_load_b128(wr[m], w_voff, ch * 64, 0);
+      R.sc[m] = __builtin_amdgcn_raw_buffer_load_b16(sr[m], s_voff, ch * (BITS == 4 ? 4 : 2), 0);
+    }
+  };
+
+  // the weight stream does not depend on the tokens: start it before anything else
+  Regs ring[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (ch0 + d < ch1) issue(ch0 + d, ring[d]);
+
+  const int64_t r0 = a.row_offsets[e];
+  const int cnt = (int)(a.row_offsets[e + 1] - a.row_offsets[e]);
+  const int xstride = x_stride_bytes(K);
+  const uint32_t nib_mask = opaque_reg(0x000f000fu), nib_magic = opaque_reg(0x43004300u);  // q -> bf16 128 + q
+  const int gpad = gpad_of(K), gstride = gsum_stride_bytes(K);
+
+  extern __shared__ __align__(16) unsigned char lds[];
+  unsigned char *lds_x = lds;
+  unsigned char *lds_ghi = lds + (tt + 1) * xstride;  // [16][gstride] bf16 high parts of the group sums
+  unsigned char *lds_glo = lds_ghi + 16 * gstride;    // low parts
   __shared__ float red[KW > 1 ? KW : 1][KW > 1 ? NW : 1][NM][4][KW > 1 ? 64 : 1];
 
-  for (int t0 = 0; t0 < cnt; t0 += TT) {
-    // activation row of this lane (A operand)
-    const int ts = BITS == 4 ? (c & 7) : c;
-    bool a_on = (t0 + ts < cnt);
-    if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
-    const uint16_t *xrow = a.x;
-    if (a_on) {
-      const int64_t r = r0 + t0 + ts;
-      const int64_t src = a.src_rows ? (int64_t)a.src_rows[r] : r;
-      xrow = a.x + src * K;
+  // zero row and zero group sums (rows that carry no token stay zero for the whole launch)
+  for (int i = threadIdx.x; i < xstride / 16; i += 256)
+    *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
+  for (int i = threadIdx.x; i < 2 * 16 * gstride / 16; i += 256)
+    *reinterpret_cast<uint4 *>(lds_ghi + i * 16) = make_uint4(0, 0, 0, 0);
+
+  for (int t0 = 0; t0 < cnt; t0 += tt) {
+    const int nt = cnt - t0 < tt ? cnt - t0 : tt;  // tokens of this tile
+    __syncthreads();  // zero fill done / every wave is done reading the previous tile
+    if (t0 > 0) {
+#pragma unroll
+      for (int d = 0; d < D; ++d)
+        if (ch0 + d < ch1) issue(ch0 + d, ring[d]);
     }
+    // stage the tile's activation rows in LDS (4-bit: each 8-block stored as the pairs
+    // (x0,x4)(x1,x5)(x2,x6)(x3,x7) the nibble unpacking produces) and the per-group sums of x.
+    // Rows past nt are never read (their lanes read the zero row); their group sums are cleared.
+    if (t0 > 0 && nt < tt)
+      for (int i = threadIdx.x; i < (tt - nt) * groups_per_row; i += 256) {
+        const int ts = nt + i / groups_per_row, g = i % groups_per_row;
+        *reinterpret_cast<uint16_t *>(lds_ghi + ts * gstride + g * 2) = 0;
+        *reinterpret_cast<uint16_t *>(lds_glo + ts * gstride + g * 2) = 0;
+      }
+    for (int i0 = 0; i0 < nt * (K / 8); i0 += 256) {
+      const int i = i0 + threadIdx.x;
+      const int ts = i / (K / 8), blk = i % (K / 8);
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (ts < nt) {
+        const int64_t r = r0 + t0 + ts;
+        const int64_t src = a.src_rows ? (int64_t)a.src_rows[r] : r;
+        v = *reinterpret_cast<const uint4 *>(a.x + src * K + blk * 8);
+      }
+      float sum = ((bf16lo_to_f32(v.x) + bf16hi_to_f32(v.x)) + (bf16lo_to_f32(v.y) + bf16hi_to_f32(v.y))) +
+                  ((bf16lo_to_f32(v.z) + bf16hi_to_f32(v.z)) + (bf16lo_to_f32(v.w) + bf16hi_to_f32(v.w)));
+      sum += __shfl_xor(sum, 1, kWave);
+      sum += __shfl_xor(sum, 2, kWave);
+      sum += __shfl_xor(sum, 4, kWave);
+      if (ts < nt) {
+        if constexpr (BITS == 4) {
+          uint4 p;
+          p.x = (v.x & 0xffffu) | (v.z << 16);
+          p.y = (v.x >> 16) | (v.z & 0xffff0000u);
+          p.z = (v.y & 0xffffu) | (v.w << 16);
+          p.w = (v.y >> 16) | (v.w & 0xffff0000u);
+          v = p;
+        }
+        *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = v;
+        if ((blk & 7) == 0) {
+          const uint32_t hi = cvt_pk_bf16(sum, 0.f) & 0xffffu;
+          const uint32_t lo = cvt_pk_bf16(sum - bf16lo_to_f32(hi), 0.f) & 0xffffu;
+          *reinterpret_cast<uint16_t *>(lds_ghi + ts * gstride + (blk >> 3) * 2) = (uint16_t)hi;
+          *reinterpret_cast<uint16_t *>(lds_glo + ts * gstride + (blk >> 3) * 2) = (uint16_t)lo;
+        }
+      }
+    }
+    __syncthreads();
+
+    // activation row of this lane (A operand); lanes without data read the zero row
+    const int ts = BITS == 4 ? (c & 7) : c;
+    bool a_on = ts < nt;
+    if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
+    const unsigned char *xl = lds_x + (a_on ? ts : tt) * xstride + kb * (CH / 4) * 2;
 
     f32x4_t tot[NM];
 #pragma unroll
     for (int m = 0; m < NM; ++m) tot[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int ch = wk; ch < nchunks; ch += KW) {
-      const int kbase = ch * CH + kb * (CH / 4);  // first code of this lane
-      const bool k_ok = kbase < K;
-      uint4 q[NM];
+    // bias term sum_g b_g * (sum_{c in g} x_c) as a small bf16 product over the group index,
+    // done once per row tile by the first K-split wave: A = group sums (hi + lo), B = biases
+    // (4-bit: b - 128 s, because the codes are fed as 128 + q), both split hi / lo.
+    if (wk == 0) {
+      for (int g0 = 0; g0 < gpad; g0 += 32) {
+        const uint4 ahi = *reinterpret_cast<const uint4 *>(lds_ghi + c * gstride + (g0 + kb * 8) * 2);
+        const uint4 alo = *reinterpret_cast<const uint4 *>(lds_glo + c * gstride + (g0 + kb * 8) * 2);
+        const uint32_t Ahi[4] = {ahi.x, ahi.y, ahi.z, ahi.w}, Alo[4] = {alo.x, alo.y, alo.z, alo.w};
 #pragma unroll
-      for (int m = 0; m < NM; ++m) {
-        q[m] = make_uint4(0, 0, 0, 0);
-        if (k_ok && tile_ok) q[m] = *reinterpret_cast<const uint4 *>(wp[m] + kbase * BITS / 32);
+        for (int m = 0; m < NM; ++m) {
+          const u32x4_t bq = __builtin_amdgcn_raw_buffer_load_b128(br[m], g_voff + (g0 + kb * 8) * 2, 0, 0);
+          u32x4_t sq = {0, 0, 0, 0};
+          if constexpr (BITS == 4)
+            sq = __builtin_amdgcn_raw_buffer_load_b128(sr[m], g_voff + (g0 + kb * 8) * 2, 0, 0);
+          uint32_t Bhi[4], Blo[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float b0 = bf16lo_to_f32(bq[i]), b1 = bf16hi_to_f32(bq[i]);
+            if constexpr (BITS == 4) {
+              b0 = __builtin_fmaf(-128.0f, bf16lo_to_f32(sq[i]), b0);
+              b1 = __builtin_fmaf(-128.0f, bf16hi_to_f32(sq[i]), b1);
+            }
+            Bhi[i] = cvt_pk_bf16(b0, b1);
+            Blo[i] = cvt_pk_bf16(b0 - bf16lo_to_f32(Bhi[i]), b1 - bf16hi_to_f32(Bhi[i]));
+          }
+          tot[m] = mfma16(Ahi, Bhi, tot[m]);
+          tot[m] = mfma16(Alo, Bhi, tot[m]);
+          tot[m] = mfma16(Ahi, Blo, tot[m]);
+        }
       }
+    }
+
+    // one chunk: MFMAs on raw codes, then the group scale applied to the fp32 group sums
+    auto compute = [&](int ch, const Regs &R) {
       uint4 xv[XV];
 #pragma unroll
-      for (int i = 0; i < XV; ++i) {
-        xv[i] = make_uint4(0, 0, 0, 0);
-        if (a_on && k_ok) xv[i] = *reinterpret_cast<const uint4 *>(xrow + kbase + i * 8);
-      }
-      // scale / bias of the group this lane's D rows belong to
-      const int g = BITS == 4 ? ch * 2 + (kb >> 1) : ch;
-      float sc[NM], bi[NM];
-#pragma unroll
-      for (int m = 0; m < NM; ++m) {
-        sc[m] = 0.f;
-        bi[m] = 0.f;
-        if (g < groups_per_row && tile_ok) {
-          sc[m] = bf16_to_f32(sp[m][g]);
-          bi[m] = bf16_to_f32(bp[m][g]);
-        }
-        if constexpr (BITS == 4) bi[m] = __builtin_fmaf(-128.0f, sc[m], bi[m]);
-      }
-
-      f32x4_t acc[NM], xs = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl + ch * CH * 2 + i * 16);
+      f32x4_t acc[NM];
 #pragma unroll
       for (int m = 0; m < NM; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
       if constexpr (BITS == 4) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          const uint4 v = xv[s];
-          uint32_t av[4];
-          av[0] = (v.x & 0xffffu) | (v.z << 16);
-          av[1] = (v.x >> 16) | (v.z & 0xffff0000u);
-          av[2] = (v.y & 0xffffu) | (v.w << 16);
-          av[3] = (v.y >> 16) | (v.w & 0xffff0000u);
-          xs = mfma16(av, ones, xs);
+          const uint32_t av[4] = {xv[s].x, xv[s].y, xv[s].z, xv[s].w};
 #pragma unroll
           for (int m = 0; m < NM; ++m) {
-            const uint32_t w = s == 0 ? q[m].x : s == 1 ? q[m].y : s == 2 ? q[m].z : q[m].w;
+            const uint32_t w = R.q[m][s];
             uint32_t bv[4];
-            bv[0] = (w & 0x000f000fu) | 0x43004300u;
-            bv[1] = ((w >> 4) & 0x000f000fu) | 0x43004300u;
-            bv[2] = ((w >> 8) & 0x000f000fu) | 0x43004300u;
-            bv[3] = ((w >> 12) & 0x000f000fu) | 0x43004300u;
+            bv[0] = and_or(w, nib_mask, nib_magic);
+            bv[1] = and_or(w >> 4, nib_mask, nib_magic);
+            bv[2] = and_or(w >> 8, nib_mask, nib_magic);
+            bv[3] = and_or(w >> 12, nib_mask, nib_magic);
             acc[m] = mfma16(av, bv, acc[m]);
           }
         }
       } else {
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-          const uint4 v = xv[s];
-          const uint32_t av[4] = {v.x, v.y, v.z, v.w};
-          xs = mfma16(av, ones, xs);
+          const uint32_t av[4] = {xv[s].x, xv[s].y, xv[s].z, xv[s].w};
 #pragma unroll
           for (int m = 0; m < NM; ++m) {
-            const uint32_t wA = s == 0 ? q[m].x : q[m].z, wB = s == 0 ? q[m].y : q[m].w;
+            const uint32_t wA = R.q[m][2 * s], wB = R.q[m][2 * s + 1];
             uint32_t bv[4];
             bv[0] = (__float_as_uint((float)(wA & 0xffu)) >> 16) |
                     (__float_as_uint((float)((wA >> 8) & 0xffu)) & 0xffff0000u);
@@ -179,10 +307,23 @@ __global__ __launch_bounds__(256) void qmm_small_kernel(GroupedArgs a) {
         }
       }
 #pragma unroll
-      for (int m = 0; m < NM; ++m)
+      for (int m = 0; m < NM; ++m) {
+        const float sc = bf16lo_to_f32(R.sc[m]);
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          tot[m][r] += sc[m] * acc[m][r] + bi[m] * xs[r];
+        for (int r = 0; r < 4; ++r) tot[m][r] += sc * acc[m][r];
+      }
+    };
+
+    // D chunks in flight: slot d is refilled as soon as its chunk has been consumed
+    for (int base = ch0; base < ch1; base += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int ch = base + d;
+        if (ch < ch1) {
+          compute(ch, ring[d]);
+          if (ch + D < ch1) issue(ch + D, ring[d]);  // refill the slot just consumed
+        }
+      }
     }
 
     if constexpr (BITS == 4) {  // rows 8-15 (second group of each chunk) onto rows 0-7
@@ -201,7 +342,6 @@ __global__ __launch_bounds__(256) void qmm_small_kernel(GroupedArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) res[m][r] = tot[m][r];
     } else {
-      __syncthreads();  // the previous token tile's readers are done with the buffer
 #pragma unroll
       for (int m = 0; m < NM; ++m)
 #pragma unroll
@@ -218,18 +358,18 @@ __global__ __launch_bounds__(256) void qmm_small_kernel(GroupedArgs a) {
         }
     }
 
-    // epilogue: one wave per row tile writes TT x 16 outputs
+    // epilogue: one wave per row tile writes nt x 16 outputs
     if (wk == 0 && tile_ok && lane < LR) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int slot = BITS == 4 ? 4 * (kb & 1) + r : 4 * kb + r;
-        if (t0 + slot < cnt) {
+        if (slot < nt) {
           const int64_t rr = r0 + t0 + slot;
           const int64_t dst = a.dst_rows ? (int64_t)a.dst_rows[rr] : rr;
           float v;
           if constexpr (GLU) v = silu_mul(res[0][r], res[1][r]);
           else v = res[0][r];
-          a.y[dst * N + n] = f32_to_bf16(v);
+          a.y[dst * N + n] = (uint16_t)(cvt_pk_bf16(v, 0.f) & 0xffffu);
         }
       }
     }
@@ -238,17 +378,25 @@ __global__ __launch_bounds__(256) void qmm_small_kernel(GroupedArgs a) {
 
 template <int BITS, bool GLU>
 static void launch_small(const GroupedArgs &a, hipStream_t st) {
+  constexpr int TT = BITS == 4 ? 8 : 16;  // token slots of one MFMA tile
+  // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
+  int tt = TT;
+  if (a.max_rows_per_expert < tt) tt = (int)a.max_rows_per_expert;
+  const size_t lds_budget = 60 * 1024;
+  while (tt > 1 && small_lds_bytes(a.K, tt) > lds_budget) --tt;
+  const size_t lds = small_lds_bytes(a.K, tt);
   // split K over the 4 waves of a block when there are too few row tiles to fill the chip
   const int64_t tiles = (int64_t)(a.N / 16) * a.max_active;
-  const int chunks = (a.K + (BITS == 4 ? 127 : 63)) / (BITS == 4 ? 128 : 64);
+  const int chunks = a.K / (BITS == 4 ? 128 : 64);
   int kw = 1;
-  if (tiles < 8192 && chunks >= 8) kw = 4;
-  else if (tiles < 16384 && chunks >= 4) kw = 2;
+  if (tiles < 4096 && chunks >= 8) kw = 4;
+  else if (tiles < 8192 && chunks >= 4) kw = 2;
+  if (const char *env = getenv("MI_MOE_KW")) kw = atoi(env);
   const int nw = 4 / kw;
   dim3 grid((unsigned)((a.N + 16 * nw - 1) / (16 * nw)), (unsigned)a.max_active);
-  if (kw == 4) qmm_small_kernel<BITS, GLU, 4><<<grid, 256, 0, st>>>(a);
-  else if (kw == 2) qmm_small_kernel<BITS, GLU, 2><<<grid, 256, 0, st>>>(a);
-  else qmm_small_kernel<BITS, GLU, 1><<<grid, 256, 0, st>>>(a);
+  if (kw == 4) qmm_small_kernel<BITS, GLU, 4><<<grid, 256, lds, st>>>(a, tt);
+  else if (kw == 2) qmm_small_kernel<BITS, GLU, 2><<<grid, 256, lds, st>>>(a, tt);
+  else qmm_small_kernel<BITS, GLU, 1><<<grid, 256, lds, st>>>(a, tt);
 }
 
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {

@@ -114,3 +114,16 @@ class SparseMoeBlock:
         return (out, dbg) if debug else out
 
     __call__ = forward
+
+    def forward_timed(self, x, out=None):
+        """One forward with HIP events between the stages; returns (out, stage_ms list)."""
+        _need(x, torch.bfloat16, "x")
+        x2 = x.reshape(-1, self.config.hidden)
+        T = x2.shape[0]
+        if out is None:
+            out = torch.empty_like(x2)
+        ws = self.reserve(max(T, 1))
+        ms = (C.c_float * capi.N_STAGES)()
+        check(self._lib.mi_moe_forward_timed(self._handle, _ptr(x2), T, _ptr(out), _ptr(ws), ws.numel(),
+                                             _stream(), ms))
+        return out.reshape(x.shape), list(ms)

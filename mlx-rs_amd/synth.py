@@ -22,13 +22,18 @@ CONFIGS = {
 }
 
 
+def _randn(shape, gen, device):
+    """Standard normal fp32 on `device`; drawn where the generator lives (CPU by default)."""
+    return torch.randn(shape, generator=gen, dtype=torch.float32, device=gen.device).to(device)
+
+
 def _bank(cfg, n_out, n_in, gen, device, std=0.02):
     E = cfg.n_experts
     w = torch.empty((E, n_out, n_in * cfg.bits // 32), dtype=torch.int32, device=device)
     s = torch.empty((E, n_out, n_in // cfg.group_size), dtype=torch.bfloat16, device=device)
     b = torch.empty_like(s)
     for e in range(E):
-        dense = (torch.randn((n_out, n_in), generator=gen, dtype=torch.float32) * std).to(device)
+        dense = _randn((n_out, n_in), gen, device) * std
         q, sc, bi = ops.quantize(dense, cfg.group_size, cfg.bits)
         w[e], s[e], b[e] = q, sc, bi
     return QuantizedSwitchLinear(w, s, b)
@@ -40,11 +45,11 @@ def zipf_bias(n_experts, s, seed):
     return (-s * torch.log(rank)).to(torch.float32)
 
 
-def make_block(cfg, seed=0, device="cuda", zipf_s=None):
-    """A SparseMoeBlock with seeded synthetic weights on ``device``."""
-    gen = torch.Generator().manual_seed(seed)
-    router = (torch.randn((cfg.n_experts, cfg.hidden), generator=gen, dtype=torch.float32) * 0.02)
-    router = router.to(torch.bfloat16).to(device)
+def make_block(cfg, seed=0, device="cuda", zipf_s=None, gen_device="cpu"):
+    """A SparseMoeBlock with seeded synthetic weights on ``device``.  gen_device="cuda" draws
+    the dense weights on the GPU (fast; the bytes then depend on the GPU's generator)."""
+    gen = torch.Generator(device=gen_device).manual_seed(seed)
+    router = (_randn((cfg.n_experts, cfg.hidden), gen, device) * 0.02).to(torch.bfloat16)
     gate = _bank(cfg, cfg.intermediate, cfg.hidden, gen, device)
     up = _bank(cfg, cfg.intermediate, cfg.hidden, gen, device)
     down = _bank(cfg, cfg.hidden, cfg.intermediate, gen, device)

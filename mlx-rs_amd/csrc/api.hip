@@ -84,7 +84,7 @@ struct ForwardWs {
   uint16_t *logits;
   uint32_t *topk_idx;
   uint16_t *topk_w;
-  uint32_t *counts, *offsets, *active, *n_active, *perm, *inv_perm, *src_of;
+  uint32_t *counts, *offsets, *work, *perm, *inv_perm, *src_of;
   void *disp_scratch;
   uint16_t *hh, *y;
   size_t bytes;
@@ -99,8 +99,7 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.topk_w = cv.take<uint16_t>((size_t)P);
   f.counts = cv.take<uint32_t>(c.n_experts);
   f.offsets = cv.take<uint32_t>(c.n_experts + 1);
-  f.active = cv.take<uint32_t>(c.n_experts);
-  f.n_active = cv.take<uint32_t>(1);
+  f.work = cv.take<uint32_t>((size_t)c.n_experts * 16);
   f.perm = cv.take<uint32_t>((size_t)P);
   f.inv_perm = cv.take<uint32_t>((size_t)P);
   f.src_of = cv.take<uint32_t>((size_t)P);
@@ -192,13 +191,11 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
   MI_STAGE_DONE();
   MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
-                         f.src_of, f.active, f.n_active, f.disp_scratch, st));
+                         f.src_of, f.work, f.disp_scratch, st));
   MI_STAGE_DONE();
   const int max_active = (int)(P < c.n_experts ? P : c.n_experts);
   GroupedArgs a{};
-  a.row_offsets = f.offsets;
-  a.active = f.active;
-  a.n_active = f.n_active;
+  a.work = f.work;
   a.max_active = max_active;
   a.bits = c.bits;
   a.total_rows = P;
@@ -206,6 +203,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
   a.x = x;
   a.src_rows = f.src_of;
+  a.src_in_work = true;
   a.dst_rows = nullptr;
   a.w0 = h->w.gate.w; a.s0 = h->w.gate.scales; a.b0 = h->w.gate.biases;
   a.w1 = h->w.up.w;   a.s1 = h->w.up.scales;   a.b1 = h->w.up.biases;
@@ -217,6 +215,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   // down: rows read in sorted order, written back in (token, slot) order
   a.x = f.hh;
   a.src_rows = nullptr;
+  a.src_in_work = false;
   a.dst_rows = f.perm;
   a.w0 = h->w.down.w; a.s0 = h->w.down.scales; a.b0 = h->w.down.biases;
   a.w1 = nullptr; a.s1 = a.b1 = nullptr;
@@ -302,7 +301,7 @@ int mi_moe_dispatch_workspace_size(int32_t n_experts, int64_t P, size_t *bytes) 
   if (!bytes) return fail("dispatch_workspace_size: bytes is NULL");
   if (n_experts < 1 || n_experts > 512 || P < 0) return fail("dispatch_workspace_size: bad arguments");
   // scratch + counts/offsets/active/n_active stand-ins for outputs the caller leaves NULL
-  *bytes = align_up(dispatch_workspace_bytes(n_experts, P)) + 4 * align_up((size_t)(n_experts + 1) * 4) + 256;
+  *bytes = align_up(dispatch_workspace_bytes(n_experts, P)) + 256;
   return 0;
 }
 
@@ -318,11 +317,9 @@ int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts
   if (!workspace || workspace_bytes < need) return fail("dispatch: workspace too small (need %zu bytes)", need);
   Carver cv(workspace);
   void *scratch = cv.take<char>(dispatch_workspace_bytes(n_experts, P));
-  uint32_t *active = cv.take<uint32_t>(n_experts + 1);
-  uint32_t *n_active = cv.take<uint32_t>(n_experts + 1);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  MI_HIP(launch_dispatch(expert_of_pair, P, n_experts, 1, counts, offsets, perm, inv_perm, nullptr, active,
-                         n_active, scratch, st));
+  MI_HIP(launch_dispatch(expert_of_pair, P, n_experts, 1, counts, offsets, perm, inv_perm, nullptr, nullptr,
+                         scratch, st));
   return 0;
 }
 
@@ -330,8 +327,8 @@ int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M
   if (!bytes) return fail("gather_qmm_workspace_size: bytes is NULL");
   if (n_experts < 1 || n_experts > 512 || n_idx < 0 || M < 1) return fail("gather_qmm_workspace_size: bad arguments");
   const int64_t rows = n_idx * M;  // perm and the (src, dst) row maps hold one entry per output row
-  *bytes = align_up(dispatch_workspace_bytes(n_experts, rows)) + 5 * align_up((size_t)(n_experts + 1) * 4) +
-           3 * align_up((size_t)rows * 4) + 256;
+  *bytes = align_up(dispatch_workspace_bytes(n_experts, rows)) + 2 * align_up((size_t)(n_experts + 1) * 4) +
+           align_up((size_t)n_experts * 64) + 3 * align_up((size_t)rows * 4) + 256;
   return 0;
 }
 
@@ -364,23 +361,19 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   void *scratch = cv.take<char>(dispatch_workspace_bytes(n_experts, rows));
   uint32_t *counts = cv.take<uint32_t>(n_experts + 1);
   uint32_t *offsets = cv.take<uint32_t>(n_experts + 1);
-  uint32_t *row_offsets = cv.take<uint32_t>(n_experts + 1);
-  uint32_t *active = cv.take<uint32_t>(n_experts + 1);
-  uint32_t *n_active = cv.take<uint32_t>(n_experts + 1);
+  uint32_t *work = cv.take<uint32_t>((size_t)n_experts * 16);
   uint32_t *perm = cv.take<uint32_t>((size_t)rows);
   uint32_t *src_rows = cv.take<uint32_t>((size_t)rows);
   uint32_t *dst_rows = cv.take<uint32_t>((size_t)rows);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  MI_HIP(launch_dispatch(rhs_indices, n_idx, n_experts, 1, counts, offsets, perm, nullptr, nullptr, active,
-                         n_active, scratch, st));
-  MI_HIP(launch_row_maps(perm, lhs_indices, offsets, n_idx, M, n_experts, src_rows, dst_rows, row_offsets, st));
+  MI_HIP(launch_dispatch(rhs_indices, n_idx, n_experts, 1, counts, offsets, perm, nullptr, nullptr, work,
+                         scratch, st));
+  MI_HIP(launch_row_maps(perm, lhs_indices, offsets, n_idx, M, n_experts, src_rows, dst_rows, work, st));
   GroupedArgs a{};
   a.x = x;
   a.src_rows = src_rows;
   a.dst_rows = dst_rows;
-  a.row_offsets = row_offsets;
-  a.active = active;
-  a.n_active = n_active;
+  a.work = work;
   a.max_active = (int)(n_idx < n_experts ? n_idx : n_experts);
   a.w0 = w; a.s0 = scales; a.b0 = biases;
   a.y = y;

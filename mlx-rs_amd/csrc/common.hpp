@@ -88,11 +88,10 @@ __device__ __forceinline__ float wave_max_f32(float v) {
 struct GroupedArgs {
   const uint16_t *x;        // bf16 rows of length K
   const uint32_t *src_rows; // x row of sorted row r, or nullptr = r
+  bool src_in_work;         // the records' inline source rows equal src_rows (saves a dependent load)
   const uint32_t *dst_rows; // output row of sorted row r, or nullptr = r
-  const uint32_t *row_offsets; // [E+1] first sorted row of each expert
-  const uint32_t *active;      // [n_active] expert ids with at least one row
-  const uint32_t *n_active;    // device scalar
-  int max_active;              // upper bound of *n_active known on the host
+  const uint32_t *work;        // 16-word records {expert, first row, rows, has_src, src[12]}, count 0 = end
+  int max_active;              // upper bound of the number of records known on the host
   const uint32_t *w0, *w1;     // packed weights [E,N,K*bits/32]; w1 only for GLU
   const uint16_t *s0, *b0, *s1, *b1;
   uint16_t *y;                 // bf16 [rows, N]
@@ -108,12 +107,11 @@ hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k,
 size_t dispatch_workspace_bytes(int E, int64_t P);
 hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
                            uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                           uint32_t *src_of, uint32_t *active, uint32_t *n_active,
-                           void *scratch, hipStream_t st);
+                           uint32_t *src_of, uint32_t *work, void *scratch, hipStream_t st);
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
-                           uint32_t *row_offsets, hipStream_t st);
+                           uint32_t *work, hipStream_t st);
 hipError_t launch_swiglu(const uint16_t *g, const uint16_t *u, int64_t n, uint16_t *out,
                          hipStream_t st);
 hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,

@@ -90,25 +90,20 @@ __device__ void scatter_range(const uint32_t *__restrict__ flat, int64_t j0, int
   }
 }
 
-// counts -> offsets, active list; runs in one block.  LDS cnt[E] in, cur[E] out.
+// Work records consumed by the grouped products: one 64-byte record per expert that received
+// rows, in ascending expert order, then records with count 0 up to n_experts.
+//   [0] expert id  [1] first sorted row  [2] row count  [3] 1 if [4..15] are filled
+//   [4..15] source row (pair index / k_div) of the first 12 rows of the segment
+constexpr int kWorkWords = 16;
+constexpr int kWorkSrc = 12;
+
+// counts -> offsets and work records; runs in one block.  LDS cnt[E] in, cur[E] (offsets) out.
 __device__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E,
                               uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
-                              uint32_t *__restrict__ active, uint32_t *__restrict__ n_active) {
+                              uint32_t *__restrict__ work, uint32_t *n_active_lds) {
   __shared__ uint32_t total;
   const int tid = threadIdx.x;
   if (tid < E && counts) counts[tid] = cnt[tid];
-  // active experts in ascending order, by wave 0
-  if (tid < kWave) {
-    uint32_t base = 0;
-    for (int e0 = 0; e0 < E; e0 += kWave) {
-      const int e = e0 + tid;
-      const bool on = e < E && cnt[e] != 0u;
-      const uint64_t bm = __ballot(on);
-      if (on && active) active[base + __popcll(bm & lanemask_lt())] = (uint32_t)e;
-      base += __popcll(bm);
-    }
-    if (tid == 0 && n_active) *n_active = base;
-  }
   __syncthreads();
   block_exclusive_scan(cnt, tmp, E, &total);
   if (tid < E) {
@@ -117,6 +112,31 @@ __device__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E
   }
   if (tid == 0 && offsets) offsets[E] = total;
   __syncthreads();
+  // experts with rows, in ascending order, by wave 0
+  if (tid < kWave) {
+    uint32_t base = 0;
+    for (int e0 = 0; e0 < E; e0 += kWave) {
+      const int e = e0 + tid;
+      uint32_t c = 0;
+      if (e < E) c = (e + 1 < E ? cnt[e + 1] : total) - cnt[e];
+      const uint64_t bm = __ballot(c != 0u);
+      if (c != 0u && work) {
+        uint32_t *rec = work + (size_t)(base + __popcll(bm & lanemask_lt())) * kWorkWords;
+        rec[0] = (uint32_t)e;
+        rec[1] = cnt[e];
+        rec[2] = c;
+        rec[3] = 0u;
+      }
+      base += __popcll(bm);
+    }
+    if (work)
+      for (int sl = base + tid; sl < E; sl += kWave) {
+        work[(size_t)sl * kWorkWords + 2] = 0u;
+        work[(size_t)sl * kWorkWords + 3] = 0u;
+      }
+    if (tid == 0) *n_active_lds = base;
+  }
+  __syncthreads();
 }
 
 // ---- one block does everything (decode-sized P)
@@ -124,8 +144,9 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_single_kernel(
     const uint32_t *__restrict__ flat, int64_t P, int E, int nbits, int k_div,
     uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets, uint32_t *__restrict__ perm,
     uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of,
-    uint32_t *__restrict__ active, uint32_t *__restrict__ n_active) {
+    uint32_t *__restrict__ work) {
   extern __shared__ uint32_t lds[];
+  __shared__ uint32_t n_active;
   uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *wcnt = lds + 3 * E;
   const int tid = threadIdx.x;
   for (int i = tid; i < E; i += kDispThreads) cnt[i] = 0u;
@@ -135,8 +156,19 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_single_kernel(
     atomicAdd(&cnt[e < (uint32_t)E ? e : (uint32_t)E - 1u], 1u);
   }
   __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, active, n_active);
+  finish_counts(cnt, tmp, cur, E, counts, offsets, work, &n_active);
   scatter_range(flat, 0, P, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
+  // source rows of the first rows of every segment, so that a consumer needs one load
+  if (work) {
+    __threadfence_block();
+    __syncthreads();
+    for (int i = tid; i < (int)n_active * kWorkSrc; i += kDispThreads) {
+      uint32_t *rec = work + (size_t)(i / kWorkSrc) * kWorkWords;
+      const uint32_t j = i % kWorkSrc;
+      if (j < rec[2]) rec[4 + j] = perm[rec[1] + j] / (uint32_t)k_div;
+      if (j == 0) rec[3] = 1u;
+    }
+  }
 }
 
 // ---- three kernels for prefill-sized P: block b owns pairs [b*span, (b+1)*span)
@@ -159,9 +191,9 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(
 
 __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
     uint32_t *__restrict__ blockhist, int nb, int E, uint32_t *__restrict__ counts,
-    uint32_t *__restrict__ offsets, uint32_t *__restrict__ active,
-    uint32_t *__restrict__ n_active) {
+    uint32_t *__restrict__ offsets, uint32_t *__restrict__ work) {
   extern __shared__ uint32_t lds[];
+  __shared__ uint32_t n_active;
   uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E;
   const int tid = threadIdx.x;
   if (tid < E) {
@@ -170,7 +202,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
     cnt[tid] = run;
   }
   __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, active, n_active);
+  finish_counts(cnt, tmp, cur, E, counts, offsets, work, &n_active);
   if (tid < E) {  // blockhist[b][e] <- first sorted position of expert e for block b
     uint32_t run = cur[tid];
     for (int b = 0; b < nb; ++b) {
@@ -206,22 +238,21 @@ size_t dispatch_workspace_bytes(int E, int64_t P) {
 
 hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
                            uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                           uint32_t *src_of, uint32_t *active, uint32_t *n_active,
-                           void *scratch, hipStream_t st) {
+                           uint32_t *src_of, uint32_t *work, void *scratch, hipStream_t st) {
   int nbits = 0;
   while ((1 << nbits) < E) ++nbits;
   if (k_div < 1) k_div = 1;
   if (P <= kSingleMaxP) {
     size_t lds = (size_t)(3 + kDispWaves) * E * sizeof(uint32_t);
     dispatch_single_kernel<<<1, kDispThreads, lds, st>>>(flat, P, E, nbits, k_div, counts, offsets,
-                                                        perm, inv_perm, src_of, active, n_active);
+                                                        perm, inv_perm, src_of, work);
     return hipGetLastError();
   }
   uint32_t *blockhist = reinterpret_cast<uint32_t *>(scratch);
   const int nb = (int)((P + kSpan - 1) / kSpan);
   dispatch_hist_kernel<<<nb, kDispThreads, (size_t)E * 4, st>>>(flat, P, E, kSpan, blockhist);
   dispatch_scan_kernel<<<1, kDispThreads, (size_t)3 * E * 4, st>>>(blockhist, nb, E, counts,
-                                                                  offsets, active, n_active);
+                                                                  offsets, work);
   dispatch_scatter_kernel<<<nb, kDispThreads, (size_t)(1 + kDispWaves) * E * 4, st>>>(
       flat, P, E, nbits, k_div, kSpan, blockhist, perm, inv_perm, src_of);
   return hipGetLastError();
@@ -232,9 +263,13 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
 __global__ void row_maps_kernel(const uint32_t *__restrict__ perm, const uint32_t *__restrict__ lhs,
                                 const uint32_t *__restrict__ offsets, int64_t n_idx, int M, int E,
                                 uint32_t *__restrict__ src_rows, uint32_t *__restrict__ dst_rows,
-                                uint32_t *__restrict__ row_offsets) {
+                                uint32_t *__restrict__ work) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i <= E) row_offsets[i] = offsets[i] * (uint32_t)M;
+  if (i < E) {  // records count rows, not indices; their inline source rows are not used
+    work[i * kWorkWords + 1] *= (uint32_t)M;
+    work[i * kWorkWords + 2] *= (uint32_t)M;
+    work[i * kWorkWords + 3] = 0u;
+  }
   if (i >= n_idx * M) return;
   const int64_t q = i / M;
   const int m = (int)(i % M);
@@ -245,10 +280,10 @@ __global__ void row_maps_kernel(const uint32_t *__restrict__ perm, const uint32_
 
 hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
-                           uint32_t *row_offsets, hipStream_t st) {
-  int64_t n = n_idx * M > E + 1 ? n_idx * M : E + 1;
+                           uint32_t *work, hipStream_t st) {
+  int64_t n = n_idx * M > E ? n_idx * M : E;
   row_maps_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(perm, lhs, offsets, n_idx, M, E,
-                                                              src_rows, dst_rows, row_offsets);
+                                                              src_rows, dst_rows, work);
   return hipGetLastError();
 }
 

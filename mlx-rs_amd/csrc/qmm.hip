@@ -61,6 +61,23 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
 //
 // KW waves of a block split K chunk-wise (wave wk takes chunks wk, wk+KW, ...), the other
 // 4/KW waves take further row tiles; partial sums meet in LDS and are added in wave order.
+#ifdef MI_MOE_TRACE
+// development aid (not built by default): per-wave time stamps of the decode kernel
+__device__ unsigned long long g_trace[8 * 16384];
+#define MI_STAMP(i)                                                                          \
+  do {                                                                                       \
+    if (lane_id() == 0) {                                                                    \
+      const unsigned wid = (blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6);   \
+      if (wid < 16384) g_trace[wid * 8 + (i)] = __builtin_readcyclecounter();               \
+    }                                                                                        \
+  } while (0)
+extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), n * sizeof(unsigned long long));
+}
+#else
+#define MI_STAMP(i) do {} while (0)
+#endif
+
 #ifndef MI_MOE_RING
 #define MI_MOE_RING 4
 #endif
@@ -77,18 +94,19 @@ template <int BITS, bool GLU>
 struct ChunkRegs {
   static constexpr int NM = GLU ? 2 : 1;
   u32x4_t q[NM];    // packed codes of this lane's weight row
-  uint32_t sc[NM];  // raw bf16 scale of the group this lane's D rows belong to
 };
 
 // LDS layout of one token tile (all offsets 16-byte aligned):
-//   [0, (tt+1)*xstride)            tt staged activation rows + one all-zero row
-//   then 2 x 16 x gpad bf16        per-(token, group) sums of x, split hi / lo, rows >= nt zero
+//   [0, (tt+1)*xstride)           tt staged activation rows + one all-zero row
+//   then groups x TT fp32         sum of x over each quantisation group, per token slot
+//   then per wave, per tensor     the bf16 scales (and biases) of the wave's 16 weight rows,
+//                                 a flat copy of 16 * K/64 values (they are contiguous in memory)
 // xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
 __host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
-__host__ __device__ constexpr int gpad_of(int K) { return (K / 64 + 31) / 32 * 32; }
-__host__ __device__ constexpr int gsum_stride_bytes(int K) { return 2 * gpad_of(K) + 16; }
-__host__ __device__ constexpr size_t small_lds_bytes(int K, int tt) {
-  return (size_t)(tt + 1) * x_stride_bytes(K) + 2 * 16 * (size_t)gsum_stride_bytes(K);
+__host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }  // 16 rows x K/64 bf16
+__host__ __device__ constexpr size_t small_lds_bytes(int K, int tt, int TT, int n_tensors) {
+  return (size_t)(tt + 1) * x_stride_bytes(K) + (size_t)(K / 64) * TT * 4 +
+         (size_t)4 * n_tensors * sb_tile_bytes(K);
 }
 
 template <int BITS, bool GLU, int KW>
@@ -101,10 +119,16 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
   constexpr int D = MI_MOE_RING;                // chunks kept in flight per wave
   using Regs = ChunkRegs<BITS, GLU>;
 
-  const uint32_t n_act = *a.n_active;
-  const uint32_t e_raw = a.active[blockIdx.y];  // the list has room for every expert
-  if (blockIdx.y >= n_act) return;
-  const int e = (int)e_raw;
+  MI_STAMP(0);
+  // one 64-byte record says everything about this block's segment (uniform address: scalar loads)
+  const uint4 *recp = reinterpret_cast<const uint4 *>(a.work) + (size_t)blockIdx.y * 4;
+  const uint4 rec0 = recp[0];
+  const int e = (int)rec0.x;
+  const int64_t r0 = rec0.y;
+  const int cnt = (int)rec0.z;
+  if (cnt == 0) return;
+  const bool rec_src = a.src_in_work && rec0.w != 0u;
+  constexpr int TT = BITS == 4 ? 8 : 16;        // token slots of one MFMA tile
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction
   const int wk = wave % KW, wn = wave / KW;
@@ -133,16 +157,13 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
     br[1] = make_rsrc(a.b1 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
   }
   const uint32_t w_voff = (uint32_t)n * row_bytes + kb * 16;  // lane kb: 16 bytes of the 64-byte chunk
-  const uint32_t g_voff = (uint32_t)n * groups_per_row * 2;
-  // 4-bit: D rows 0-7 (lanes kb < 2) belong to a chunk's first group, rows 8-15 to its second
-  const uint32_t s_voff = g_voff + (BITS == 4 ? (kb >> 1) * 2 : 0);
+  const int sbt = sb_tile_bytes(K);
 
   // issue every global load of chunk ch into R
   auto issue = [&](int ch, Regs &R) {
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
       R.q[m] = __builtin_amdgcn_raw_buffer_load_b128(wr[m], w_voff, ch * 64, 0);
-      R.sc[m] = __builtin_amdgcn_raw_buffer_load_b16(sr[m], s_voff, ch * (BITS == 4 ? 4 : 2), 0);
     }
   };
 
@@ -152,23 +173,48 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
   for (int d = 0; d < D; ++d)
     if (ch0 + d < ch1) issue(ch0 + d, ring[d]);
 
-  const int64_t r0 = a.row_offsets[e];
-  const int cnt = (int)(a.row_offsets[e + 1] - a.row_offsets[e]);
+  // scales and biases of the wave's 16 rows: K/2 contiguous bytes per tensor, fetched with
+  // fully coalesced 16-byte loads now and parked in LDS (wave-private) before the chunk loop
+  constexpr int NTEN = 2 * NM;  // tensors: scales, biases (x gate, up)
+  constexpr int SBI = 2;        // 16-byte loads per lane per tensor kept in registers (K <= 4096)
+  const uint32_t sb_goff = (uint32_t)n0 * groups_per_row * 2 + lane * 16;
+  u32x4_t sbv[NTEN][SBI];
+#pragma unroll
+  for (int t = 0; t < NTEN; ++t)
+#pragma unroll
+    for (int i = 0; i < SBI; ++i)
+      if (i * 1024 < sbt)
+        sbv[t][i] = __builtin_amdgcn_raw_buffer_load_b128((t & 1) ? br[t >> 1] : sr[t >> 1], sb_goff, i * 1024, 0);
+
+  MI_STAMP(1);
   const int xstride = x_stride_bytes(K);
   const uint32_t nib_mask = opaque_reg(0x000f000fu), nib_magic = opaque_reg(0x43004300u);  // q -> bf16 128 + q
-  const int gpad = gpad_of(K), gstride = gsum_stride_bytes(K);
 
   extern __shared__ __align__(16) unsigned char lds[];
   unsigned char *lds_x = lds;
-  unsigned char *lds_ghi = lds + (tt + 1) * xstride;  // [16][gstride] bf16 high parts of the group sums
-  unsigned char *lds_glo = lds_ghi + 16 * gstride;    // low parts
+  float *lds_gs = reinterpret_cast<float *>(lds + (tt + 1) * xstride);  // [groups][TT] sums of x
+  unsigned char *lds_sb = lds + (tt + 1) * xstride + groups_per_row * TT * 4 + wave * NTEN * sbt;
+
+  // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait)
+#pragma unroll
+  for (int t = 0; t < NTEN; ++t) {
+#pragma unroll
+    for (int i = 0; i < SBI; ++i)
+      if (i * 1024 + lane * 16 < sbt)
+        *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + i * 1024 + lane * 16) = sbv[t][i];
+    for (int off = SBI * 1024 + lane * 16; off < sbt; off += 1024)  // K > 4096: the rest, synchronously
+      *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + off) = __builtin_amdgcn_raw_buffer_load_b128(
+          (t & 1) ? br[t >> 1] : sr[t >> 1], (uint32_t)n0 * groups_per_row * 2 + off, 0, 0);
+  }
+  // this lane's scale / bias of chunk 0: row c, group (4-bit) kb >> 1 of the chunk's two
+  const unsigned char *sbl = lds_sb + (c * groups_per_row + (BITS == 4 ? (kb >> 1) : 0)) * 2;
   __shared__ float red[KW > 1 ? KW : 1][KW > 1 ? NW : 1][NM][4][KW > 1 ? 64 : 1];
 
-  // zero row and zero group sums (rows that carry no token stay zero for the whole launch)
+  // zero row and zero group sums (slots that carry no token stay zero for the whole launch)
   for (int i = threadIdx.x; i < xstride / 16; i += 256)
     *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
-  for (int i = threadIdx.x; i < 2 * 16 * gstride / 16; i += 256)
-    *reinterpret_cast<uint4 *>(lds_ghi + i * 16) = make_uint4(0, 0, 0, 0);
+  for (int i = threadIdx.x; i < groups_per_row * TT / 4; i += 256)
+    *reinterpret_cast<uint4 *>(lds_gs + i * 4) = make_uint4(0, 0, 0, 0);
 
   for (int t0 = 0; t0 < cnt; t0 += tt) {
     const int nt = cnt - t0 < tt ? cnt - t0 : tt;  // tokens of this tile
@@ -182,18 +228,22 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
     // (x0,x4)(x1,x5)(x2,x6)(x3,x7) the nibble unpacking produces) and the per-group sums of x.
     // Rows past nt are never read (their lanes read the zero row); their group sums are cleared.
     if (t0 > 0 && nt < tt)
-      for (int i = threadIdx.x; i < (tt - nt) * groups_per_row; i += 256) {
-        const int ts = nt + i / groups_per_row, g = i % groups_per_row;
-        *reinterpret_cast<uint16_t *>(lds_ghi + ts * gstride + g * 2) = 0;
-        *reinterpret_cast<uint16_t *>(lds_glo + ts * gstride + g * 2) = 0;
-      }
+      for (int i = threadIdx.x; i < (tt - nt) * groups_per_row; i += 256)
+        lds_gs[(i / (tt - nt)) * TT + nt + i % (tt - nt)] = 0.f;
     for (int i0 = 0; i0 < nt * (K / 8); i0 += 256) {
       const int i = i0 + threadIdx.x;
       const int ts = i / (K / 8), blk = i % (K / 8);
       uint4 v = make_uint4(0, 0, 0, 0);
       if (ts < nt) {
         const int64_t r = r0 + t0 + ts;
-        const int64_t src = a.src_rows ? (int64_t)a.src_rows[r] : r;
+        int64_t src = r;
+        if (rec_src && t0 + ts < 12) {  // source row from the record (no dependent global load)
+          const uint4 q4 = recp[1 + ((t0 + ts) >> 2)];
+          const int j = (t0 + ts) & 3;
+          src = j == 0 ? q4.x : j == 1 ? q4.y : j == 2 ? q4.z : q4.w;
+        } else if (a.src_rows) {
+          src = a.src_rows[r];
+        }
         v = *reinterpret_cast<const uint4 *>(a.x + src * K + blk * 8);
       }
       float sum = ((bf16lo_to_f32(v.x) + bf16hi_to_f32(v.x)) + (bf16lo_to_f32(v.y) + bf16hi_to_f32(v.y))) +
@@ -211,15 +261,12 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
           v = p;
         }
         *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = v;
-        if ((blk & 7) == 0) {
-          const uint32_t hi = cvt_pk_bf16(sum, 0.f) & 0xffffu;
-          const uint32_t lo = cvt_pk_bf16(sum - bf16lo_to_f32(hi), 0.f) & 0xffffu;
-          *reinterpret_cast<uint16_t *>(lds_ghi + ts * gstride + (blk >> 3) * 2) = (uint16_t)hi;
-          *reinterpret_cast<uint16_t *>(lds_glo + ts * gstride + (blk >> 3) * 2) = (uint16_t)lo;
-        }
+        if ((blk & 7) == 0) lds_gs[(blk >> 3) * TT + ts] = sum;
       }
     }
+    MI_STAMP(2);
     __syncthreads();
+    MI_STAMP(3);
 
     // activation row of this lane (A operand); lanes without data read the zero row
     const int ts = BITS == 4 ? (c & 7) : c;
@@ -231,39 +278,10 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
 #pragma unroll
     for (int m = 0; m < NM; ++m) tot[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // bias term sum_g b_g * (sum_{c in g} x_c) as a small bf16 product over the group index,
-    // done once per row tile by the first K-split wave: A = group sums (hi + lo), B = biases
-    // (4-bit: b - 128 s, because the codes are fed as 128 + q), both split hi / lo.
-    if (wk == 0) {
-      for (int g0 = 0; g0 < gpad; g0 += 32) {
-        const uint4 ahi = *reinterpret_cast<const uint4 *>(lds_ghi + c * gstride + (g0 + kb * 8) * 2);
-        const uint4 alo = *reinterpret_cast<const uint4 *>(lds_glo + c * gstride + (g0 + kb * 8) * 2);
-        const uint32_t Ahi[4] = {ahi.x, ahi.y, ahi.z, ahi.w}, Alo[4] = {alo.x, alo.y, alo.z, alo.w};
-#pragma unroll
-        for (int m = 0; m < NM; ++m) {
-          const u32x4_t bq = __builtin_amdgcn_raw_buffer_load_b128(br[m], g_voff + (g0 + kb * 8) * 2, 0, 0);
-          u32x4_t sq = {0, 0, 0, 0};
-          if constexpr (BITS == 4)
-            sq = __builtin_amdgcn_raw_buffer_load_b128(sr[m], g_voff + (g0 + kb * 8) * 2, 0, 0);
-          uint32_t Bhi[4], Blo[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float b0 = bf16lo_to_f32(bq[i]), b1 = bf16hi_to_f32(bq[i]);
-            if constexpr (BITS == 4) {
-              b0 = __builtin_fmaf(-128.0f, bf16lo_to_f32(sq[i]), b0);
-              b1 = __builtin_fmaf(-128.0f, bf16hi_to_f32(sq[i]), b1);
-            }
-            Bhi[i] = cvt_pk_bf16(b0, b1);
-            Blo[i] = cvt_pk_bf16(b0 - bf16lo_to_f32(Bhi[i]), b1 - bf16hi_to_f32(Bhi[i]));
-          }
-          tot[m] = mfma16(Ahi, Bhi, tot[m]);
-          tot[m] = mfma16(Alo, Bhi, tot[m]);
-          tot[m] = mfma16(Ahi, Blo, tot[m]);
-        }
-      }
-    }
+    // group sums of x for this lane's 4 D rows (token slots), first group of chunk 0
+    const float *gsl = lds_gs + (BITS == 4 ? (kb >> 1) * TT + 4 * (kb & 1) : 4 * kb);
 
-    // one chunk: MFMAs on raw codes, then the group scale applied to the fp32 group sums
+    // one chunk: MFMAs on raw codes, then scale and bias applied to the fp32 group sums
     auto compute = [&](int ch, const Regs &R) {
       uint4 xv[XV];
 #pragma unroll
@@ -306,14 +324,22 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
           }
         }
       }
+      // sum_c x_c (s (128 + q_c - 128) + b) = s * acc + (b - 128 s) * sum_c x_c   (8-bit: no offset)
+      const float4 xs = *reinterpret_cast<const float4 *>(gsl + ch * (BITS == 4 ? 2 : 1) * TT);
 #pragma unroll
       for (int m = 0; m < NM; ++m) {
-        const float sc = bf16lo_to_f32(R.sc[m]);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) tot[m][r] += sc * acc[m][r];
+        const int goff = ch * (BITS == 4 ? 4 : 2);
+        const float sc = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m) * sbt + goff));
+        float bi = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m + 1) * sbt + goff));
+        if constexpr (BITS == 4) bi = __builtin_fmaf(-128.0f, sc, bi);
+        tot[m][0] += sc * acc[m][0] + bi * xs.x;
+        tot[m][1] += sc * acc[m][1] + bi * xs.y;
+        tot[m][2] += sc * acc[m][2] + bi * xs.z;
+        tot[m][3] += sc * acc[m][3] + bi * xs.w;
       }
     };
 
+    MI_STAMP(4);
     // D chunks in flight: slot d is refilled as soon as its chunk has been consumed
     for (int base = ch0; base < ch1; base += D) {
 #pragma unroll
@@ -326,6 +352,7 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
       }
     }
 
+    MI_STAMP(5);
     if constexpr (BITS == 4) {  // rows 8-15 (second group of each chunk) onto rows 0-7
 #pragma unroll
       for (int m = 0; m < NM; ++m)
@@ -381,10 +408,12 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   constexpr int TT = BITS == 4 ? 8 : 16;  // token slots of one MFMA tile
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
   int tt = TT;
+  // short segments on average: stage fewer rows, the LDS saved buys a fourth block per CU
+  if (a.total_rows <= 3 * (int64_t)a.max_active && tt > 4) tt = 4;
   if (a.max_rows_per_expert < tt) tt = (int)a.max_rows_per_expert;
   const size_t lds_budget = 60 * 1024;
-  while (tt > 1 && small_lds_bytes(a.K, tt) > lds_budget) --tt;
-  const size_t lds = small_lds_bytes(a.K, tt);
+  while (tt > 1 && small_lds_bytes(a.K, tt, TT, GLU ? 4 : 2) > lds_budget) --tt;
+  const size_t lds = small_lds_bytes(a.K, tt, TT, GLU ? 4 : 2);
   // split K over the 4 waves of a block when there are too few row tiles to fill the chip
   const int64_t tiles = (int64_t)(a.N / 16) * a.max_active;
   const int chunks = a.K / (BITS == 4 ? 128 : 64);

@@ -66,7 +66,7 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
 __device__ unsigned long long g_trace[8 * 16384];
 #define MI_STAMP(i)                                                                          \
   do {                                                                                       \
-    if (lane_id() == 0) {                                                                    \
+    if (GLU && lane_id() == 0) {                                                             \
       const unsigned wid = (blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6);   \
       if (wid < 16384) g_trace[wid * 8 + (i)] = __builtin_readcyclecounter();               \
     }                                                                                        \
@@ -127,6 +127,7 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
   const int64_t r0 = rec0.y;
   const int cnt = (int)rec0.z;
   if (cnt == 0) return;
+  MI_STAMP(6);
   const bool rec_src = a.src_in_work && rec0.w != 0u;
   constexpr int TT = BITS == 4 ? 8 : 16;        // token slots of one MFMA tile
   const int lane = lane_id();
@@ -230,38 +231,43 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
     if (t0 > 0 && nt < tt)
       for (int i = threadIdx.x; i < (tt - nt) * groups_per_row; i += 256)
         lds_gs[(i / (tt - nt)) * TT + nt + i % (tt - nt)] = 0.f;
-    for (int i0 = 0; i0 < nt * (K / 8); i0 += 256) {
-      const int i = i0 + threadIdx.x;
-      const int ts = i / (K / 8), blk = i % (K / 8);
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (ts < nt) {
-        const int64_t r = r0 + t0 + ts;
-        int64_t src = r;
-        if (rec_src && t0 + ts < 12) {  // source row from the record (no dependent global load)
-          const uint4 q4 = recp[1 + ((t0 + ts) >> 2)];
-          const int j = (t0 + ts) & 3;
-          src = j == 0 ? q4.x : j == 1 ? q4.y : j == 2 ? q4.z : q4.w;
-        } else if (a.src_rows) {
-          src = a.src_rows[r];
+    // wave w stages token slots w, w+4, ...: the source row is wave-uniform (read from the
+    // record through the scalar cache) and every load of a row is issued before the first use
+    for (int ts = wave; ts < nt; ts += 4) {
+      const int64_t r = r0 + t0 + ts;
+      int64_t src = r;
+      if (rec_src && t0 + ts < 12) src = a.work[(size_t)blockIdx.y * 16 + 4 + t0 + ts];
+      else if (a.src_rows) src = a.src_rows[r];
+      const uint16_t *xr = a.x + src * K;
+      for (int b0 = 0; b0 < K / 8; b0 += 256) {
+        uint4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int blk = b0 + j * 64 + lane;
+          v[j] = make_uint4(0, 0, 0, 0);
+          if (blk < K / 8) v[j] = *reinterpret_cast<const uint4 *>(xr + blk * 8);
         }
-        v = *reinterpret_cast<const uint4 *>(a.x + src * K + blk * 8);
-      }
-      float sum = ((bf16lo_to_f32(v.x) + bf16hi_to_f32(v.x)) + (bf16lo_to_f32(v.y) + bf16hi_to_f32(v.y))) +
-                  ((bf16lo_to_f32(v.z) + bf16hi_to_f32(v.z)) + (bf16lo_to_f32(v.w) + bf16hi_to_f32(v.w)));
-      sum += __shfl_xor(sum, 1, kWave);
-      sum += __shfl_xor(sum, 2, kWave);
-      sum += __shfl_xor(sum, 4, kWave);
-      if (ts < nt) {
-        if constexpr (BITS == 4) {
-          uint4 p;
-          p.x = (v.x & 0xffffu) | (v.z << 16);
-          p.y = (v.x >> 16) | (v.z & 0xffff0000u);
-          p.z = (v.y & 0xffffu) | (v.w << 16);
-          p.w = (v.y >> 16) | (v.w & 0xffff0000u);
-          v = p;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int blk = b0 + j * 64 + lane;
+          const uint4 w = v[j];
+          float sum = ((bf16lo_to_f32(w.x) + bf16hi_to_f32(w.x)) + (bf16lo_to_f32(w.y) + bf16hi_to_f32(w.y))) +
+                      ((bf16lo_to_f32(w.z) + bf16hi_to_f32(w.z)) + (bf16lo_to_f32(w.w) + bf16hi_to_f32(w.w)));
+          sum += __shfl_xor(sum, 1, kWave);
+          sum += __shfl_xor(sum, 2, kWave);
+          sum += __shfl_xor(sum, 4, kWave);
+          if (blk < K / 8) {
+            uint4 p = w;
+            if constexpr (BITS == 4) {
+              p.x = (w.x & 0xffffu) | (w.z << 16);
+              p.y = (w.x >> 16) | (w.z & 0xffff0000u);
+              p.z = (w.y & 0xffffu) | (w.w << 16);
+              p.w = (w.y >> 16) | (w.w & 0xffff0000u);
+            }
+            *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = p;
+            if ((blk & 7) == 0) lds_gs[(blk >> 3) * TT + ts] = sum;
+          }
         }
-        *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = v;
-        if ((blk & 7) == 0) lds_gs[(blk >> 3) * TT + ts] = sum;
       }
     }
     MI_STAMP(2);
@@ -332,10 +338,10 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
         const float sc = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m) * sbt + goff));
         float bi = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m + 1) * sbt + goff));
         if constexpr (BITS == 4) bi = __builtin_fmaf(-128.0f, sc, bi);
-        tot[m][0] += sc * acc[m][0] + bi * xs.x;
-        tot[m][1] += sc * acc[m][1] + bi * xs.y;
-        tot[m][2] += sc * acc[m][2] + bi * xs.z;
-        tot[m][3] += sc * acc[m][3] + bi * xs.w;
+        tot[m][0] = __builtin_fmaf(sc, acc[m][0], __builtin_fmaf(bi, xs.x, tot[m][0]));
+        tot[m][1] = __builtin_fmaf(sc, acc[m][1], __builtin_fmaf(bi, xs.y, tot[m][1]));
+        tot[m][2] = __builtin_fmaf(sc, acc[m][2], __builtin_fmaf(bi, xs.z, tot[m][2]));
+        tot[m][3] = __builtin_fmaf(sc, acc[m][3], __builtin_fmaf(bi, xs.w, tot[m][3]));
       }
     };
 

@@ -84,7 +84,8 @@ struct ForwardWs {
   uint16_t *logits;
   uint32_t *topk_idx;
   uint16_t *topk_w;
-  uint32_t *counts, *offsets, *work, *perm, *inv_perm, *src_of;
+  uint32_t *counts, *offsets, *work, *mtiles, *perm, *inv_perm, *src_of;
+  int max_mtiles;
   void *disp_scratch;
   uint16_t *hh, *y;
   size_t bytes;
@@ -100,6 +101,9 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.counts = cv.take<uint32_t>(c.n_experts);
   f.offsets = cv.take<uint32_t>(c.n_experts + 1);
   f.work = cv.take<uint32_t>((size_t)c.n_experts * 16);
+  // M tiles of the tiled kernel: at most one partial tile per long segment plus P / tile full ones
+  f.max_mtiles = P >= kBigThreshold ? (int)(P / kBigTileM + (P / kBigThreshold < c.n_experts ? P / kBigThreshold : c.n_experts)) : 0;
+  f.mtiles = cv.take<uint32_t>(4 + (size_t)f.max_mtiles * 4);
   f.perm = cv.take<uint32_t>((size_t)P);
   f.inv_perm = cv.take<uint32_t>((size_t)P);
   f.src_of = cv.take<uint32_t>((size_t)P);
@@ -191,12 +195,14 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
   MI_STAGE_DONE();
   MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
-                         f.src_of, f.work, f.disp_scratch, st));
+                         f.src_of, f.work, f.max_mtiles ? f.mtiles : nullptr, kBigThreshold, f.disp_scratch, st));
   MI_STAGE_DONE();
   const int max_active = (int)(P < c.n_experts ? P : c.n_experts);
   GroupedArgs a{};
   a.work = f.work;
   a.max_active = max_active;
+  a.mtiles = f.max_mtiles ? f.mtiles : nullptr;
+  a.max_mtiles = f.max_mtiles;
   a.bits = c.bits;
   a.total_rows = P;
   a.max_rows_per_expert = T;  // a token picks an expert at most once
@@ -319,7 +325,7 @@ int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts
   void *scratch = cv.take<char>(dispatch_workspace_bytes(n_experts, P));
   hipStream_t st = static_cast<hipStream_t>(stream);
   MI_HIP(launch_dispatch(expert_of_pair, P, n_experts, 1, counts, offsets, perm, inv_perm, nullptr, nullptr,
-                         scratch, st));
+                         nullptr, 0, scratch, st));
   return 0;
 }
 
@@ -367,7 +373,7 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   uint32_t *dst_rows = cv.take<uint32_t>((size_t)rows);
   hipStream_t st = static_cast<hipStream_t>(stream);
   MI_HIP(launch_dispatch(rhs_indices, n_idx, n_experts, 1, counts, offsets, perm, nullptr, nullptr, work,
-                         scratch, st));
+                         nullptr, 0, scratch, st));
   MI_HIP(launch_row_maps(perm, lhs_indices, offsets, n_idx, M, n_experts, src_rows, dst_rows, work, st));
   GroupedArgs a{};
   a.x = x;

@@ -7,6 +7,8 @@
 namespace mi_moe {
 
 constexpr int kWave = 64;
+constexpr int kBigThreshold = 24;  // segments with at least this many rows use the tiled kernel
+constexpr int kBigTileM = 256;     // rows per M tile of the tiled kernel
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
@@ -92,6 +94,8 @@ struct GroupedArgs {
   const uint32_t *dst_rows; // output row of sorted row r, or nullptr = r
   const uint32_t *work;        // 16-word records {expert, first row, rows, has_src, src[12]}, count 0 = end
   int max_active;              // upper bound of the number of records known on the host
+  const uint32_t *mtiles;      // M tiles of the long segments (tiled MFMA kernel), or nullptr
+  int max_mtiles;              // host upper bound of the number of M tiles
   const uint32_t *w0, *w1;     // packed weights [E,N,K*bits/32]; w1 only for GLU
   const uint16_t *s0, *b0, *s1, *b1;
   uint16_t *y;                 // bf16 [rows, N]
@@ -107,8 +111,10 @@ hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k,
 size_t dispatch_workspace_bytes(int E, int64_t P);
 hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
                            uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                           uint32_t *src_of, uint32_t *work, void *scratch, hipStream_t st);
+                           uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
+                           void *scratch, hipStream_t st);
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
+hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
                            uint32_t *work, hipStream_t st);

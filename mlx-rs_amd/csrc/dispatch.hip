@@ -97,10 +97,16 @@ __device__ void scatter_range(const uint32_t *__restrict__ flat, int64_t j0, int
 constexpr int kWorkWords = 16;
 constexpr int kWorkSrc = 12;
 
-// counts -> offsets and work records; runs in one block.  LDS cnt[E] in, cur[E] (offsets) out.
+// Long segments (at least big_thr rows, big_thr > 0) go to the tiled MFMA kernel instead: they
+// are cut into M tiles of kBigTileM rows, listed in `mtiles`:
+//   mtiles[0] = number of tiles; tile i at mtiles[4 + 4 i] = {expert id, first sorted row, rows, 0}
+
+
+// counts -> offsets, work records and M tiles; runs in one block.  LDS cnt[E] in, cur[E] out.
 __device__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E,
                               uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
-                              uint32_t *__restrict__ work, uint32_t *n_active_lds) {
+                              uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
+                              uint32_t big_thr, uint32_t *n_active_lds) {
   __shared__ uint32_t total;
   const int tid = threadIdx.x;
   if (tid < E && counts) counts[tid] = cnt[tid];
@@ -114,13 +120,15 @@ __device__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E
   __syncthreads();
   // experts with rows, in ascending order, by wave 0
   if (tid < kWave) {
-    uint32_t base = 0;
+    uint32_t base = 0, tbase = 0;
     for (int e0 = 0; e0 < E; e0 += kWave) {
       const int e = e0 + tid;
       uint32_t c = 0;
       if (e < E) c = (e + 1 < E ? cnt[e + 1] : total) - cnt[e];
-      const uint64_t bm = __ballot(c != 0u);
-      if (c != 0u && work) {
+      const bool big = mtiles && big_thr != 0u && c >= big_thr;
+      const bool small = c != 0u && !big;
+      const uint64_t bm = __ballot(small);
+      if (small && work) {
         uint32_t *rec = work + (size_t)(base + __popcll(bm & lanemask_lt())) * kWorkWords;
         rec[0] = (uint32_t)e;
         rec[1] = cnt[e];
@@ -128,13 +136,31 @@ __device__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E
         rec[3] = 0u;
       }
       base += __popcll(bm);
+      // M tiles of the long segments: exclusive scan of the tile counts over the wave
+      const uint32_t nt = big ? (c + kBigTileM - 1) / kBigTileM : 0u;
+      uint32_t incl = nt;
+      for (int d = 1; d < kWave; d <<= 1) {
+        const uint32_t v = __shfl_up(incl, d, kWave);
+        if (tid >= d) incl += v;
+      }
+      for (uint32_t i = 0; i < nt; ++i) {
+        uint32_t *rec = mtiles + 4 + (size_t)(tbase + incl - nt + i) * 4;
+        rec[0] = (uint32_t)e;
+        rec[1] = cnt[e] + i * kBigTileM;
+        rec[2] = c - i * kBigTileM < (uint32_t)kBigTileM ? c - i * kBigTileM : (uint32_t)kBigTileM;
+        rec[3] = 0u;
+      }
+      tbase += __shfl(incl, kWave - 1, kWave);
     }
     if (work)
       for (int sl = base + tid; sl < E; sl += kWave) {
         work[(size_t)sl * kWorkWords + 2] = 0u;
         work[(size_t)sl * kWorkWords + 3] = 0u;
       }
-    if (tid == 0) *n_active_lds = base;
+    if (tid == 0) {
+      *n_active_lds = base;
+      if (mtiles) mtiles[0] = tbase;
+    }
   }
   __syncthreads();
 }
@@ -144,7 +170,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_single_kernel(
     const uint32_t *__restrict__ flat, int64_t P, int E, int nbits, int k_div,
     uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets, uint32_t *__restrict__ perm,
     uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of,
-    uint32_t *__restrict__ work) {
+    uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles, uint32_t big_thr) {
   extern __shared__ uint32_t lds[];
   __shared__ uint32_t n_active;
   uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *wcnt = lds + 3 * E;
@@ -156,7 +182,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_single_kernel(
     atomicAdd(&cnt[e < (uint32_t)E ? e : (uint32_t)E - 1u], 1u);
   }
   __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, work, &n_active);
+  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, big_thr, &n_active);
   scatter_range(flat, 0, P, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
   // source rows of the first rows of every segment, so that a consumer needs one load
   if (work) {
@@ -191,7 +217,8 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(
 
 __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
     uint32_t *__restrict__ blockhist, int nb, int E, uint32_t *__restrict__ counts,
-    uint32_t *__restrict__ offsets, uint32_t *__restrict__ work) {
+    uint32_t *__restrict__ offsets, uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
+    uint32_t big_thr) {
   extern __shared__ uint32_t lds[];
   __shared__ uint32_t n_active;
   uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E;
@@ -202,7 +229,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
     cnt[tid] = run;
   }
   __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, work, &n_active);
+  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, big_thr, &n_active);
   if (tid < E) {  // blockhist[b][e] <- first sorted position of expert e for block b
     uint32_t run = cur[tid];
     for (int b = 0; b < nb; ++b) {
@@ -238,21 +265,22 @@ size_t dispatch_workspace_bytes(int E, int64_t P) {
 
 hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
                            uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                           uint32_t *src_of, uint32_t *work, void *scratch, hipStream_t st) {
+                           uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
+                           void *scratch, hipStream_t st) {
   int nbits = 0;
   while ((1 << nbits) < E) ++nbits;
   if (k_div < 1) k_div = 1;
   if (P <= kSingleMaxP) {
     size_t lds = (size_t)(3 + kDispWaves) * E * sizeof(uint32_t);
     dispatch_single_kernel<<<1, kDispThreads, lds, st>>>(flat, P, E, nbits, k_div, counts, offsets,
-                                                        perm, inv_perm, src_of, work);
+                                                        perm, inv_perm, src_of, work, mtiles, (uint32_t)big_thr);
     return hipGetLastError();
   }
   uint32_t *blockhist = reinterpret_cast<uint32_t *>(scratch);
   const int nb = (int)((P + kSpan - 1) / kSpan);
   dispatch_hist_kernel<<<nb, kDispThreads, (size_t)E * 4, st>>>(flat, P, E, kSpan, blockhist);
   dispatch_scan_kernel<<<1, kDispThreads, (size_t)3 * E * 4, st>>>(blockhist, nb, E, counts,
-                                                                  offsets, work);
+                                                                  offsets, work, mtiles, (uint32_t)big_thr);
   dispatch_scatter_kernel<<<nb, kDispThreads, (size_t)(1 + kDispWaves) * E * 4, st>>>(
       flat, P, E, nbits, k_div, kSpan, blockhist, perm, inv_perm, src_of);
   return hipGetLastError();

@@ -436,6 +436,8 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
 
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
   if (a.max_active <= 0 || a.total_rows <= 0) return hipSuccess;
+  // long segments (listed as M tiles by the dispatch) go to the tiled kernel, the rest below
+  if (hipError_t e = launch_large_qmm(a, glu, st); e != hipSuccess) return e;
   if (a.bits == 4) {
     if (glu) launch_small<4, true>(a, st);
     else launch_small<4, false>(a, st);

@@ -175,7 +175,7 @@ def route(cfg, router_w, router_bias, x):
 
 
 def dispatch(flat, E):
-    flat = _c(np.asarray(flat).reshape(-1), np.uint32)
+    flat = np.ascontiguousarray(np.asarray(flat).reshape(-1).astype(np.uint32))
     P = flat.size
     counts = np.empty(E, np.uint32)
     offsets = np.empty(E + 1, np.uint32)
@@ -191,9 +191,9 @@ def gather_qmm(x, w, s, b, lhs, rhs, bits=4, group=64, n_threads=8, want="f32"):
     s, b = _c(s, np.uint16), _c(b, np.uint16)
     xb, M, K = x.shape
     E, N = w.shape[0], w.shape[1]
-    rhs = _c(np.asarray(rhs).reshape(-1), np.uint32)
+    rhs = np.ascontiguousarray(np.asarray(rhs).reshape(-1).astype(np.uint32))
     if lhs is not None:
-        lhs = _c(np.asarray(lhs).reshape(-1), np.uint32)
+        lhs = np.ascontiguousarray(np.asarray(lhs).reshape(-1).astype(np.uint32))
     n_idx = rhs.size
     yf = np.empty((n_idx, M, N), np.float32) if want == "f32" else None
     yb = np.empty((n_idx, M, N), np.uint16) if want == "bf16" else None

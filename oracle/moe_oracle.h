@@ -16,9 +16,11 @@
  * Pinning status (what independent check each function has, tests/test_oracle_*.py):
  *   orc_quantize / orc_dequantize  pinned: reference KAT ops/quantization.rs:298-315
  *                                  (arange 128x512, group 128, bits 2/4/8: shapes +
- *                                  max error bound), |w - w_hat| <= |scale|/2, special
- *                                  groups (zero, constant, negative-dominant), packing
- *                                  order against a bit-by-bit numpy unpack.
+ *                                  max error bound), nearest-code property by brute force
+ *                                  over all codes, exact zero in groups that straddle
+ *                                  zero, special groups (zero, constant, negative-
+ *                                  dominant), packing order against a bit-by-bit numpy
+ *                                  unpack.
  *                                  The exact bits of mlx.quantize on arbitrary input
  *                                  (eps clamp, rint mode, cast timing) are
  *                                  "parity unpinned": MLX is not importable here.  They

@@ -1,0 +1,112 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports every symbol the
+header declares, and rejects bad arguments with a status and a message (never a crash), the way
+mlx-sys calls report errors to mlx-rs (mlx-rs/src/utils/guard.rs:20-49, error.rs:226-280;
+error-path tests ops/sort.rs:266-298)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import mlx_rs_amd as m
+    return m.load_library()
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "mi_moe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi_moe_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    import mlx_rs_amd as m
+    syms = header_symbols()
+    assert len(syms) >= 17
+    for s in syms:
+        assert hasattr(lib, s), f"{s} is declared in include/mi_moe.h but not exported"
+    assert sorted(m.capi.EXPORTS) == syms
+    assert lib.mi_moe_version().startswith(b"mi_moe")
+
+
+def cfg(**kw):
+    import mlx_rs_amd as m
+    base = dict(hidden=256, n_experts=8, top_k=2, intermediate=512, bits=4, group_size=64, score_mode=0)
+    base.update(kw)
+    return m.capi.Config(**base)
+
+
+@pytest.mark.parametrize("kw,needle", [
+    (dict(hidden=100), "hidden"), (dict(bits=3), "bits"), (dict(group_size=32), "group_size"),
+    (dict(top_k=9), "top_k"), (dict(top_k=0), "top_k"), (dict(n_experts=0), "n_experts"),
+    (dict(intermediate=96), "intermediate"), (dict(score_mode=7), "score_mode"),
+    (dict(hidden=192), "128"),
+])
+def test_bad_config_is_rejected_with_a_message(lib, kw, needle):
+    import mlx_rs_amd as m
+    n = C.c_size_t(12345)
+    c = cfg(**kw)
+    assert lib.mi_moe_workspace_size(C.byref(c), 4, C.byref(n)) != 0
+    assert needle in m.capi.last_error()
+    assert n.value == 12345                     # outputs untouched on failure
+    with pytest.raises(m.MoeError):
+        m.capi.check(1)
+
+
+def test_null_and_range_checks(lib):
+    import mlx_rs_amd as m
+    c = cfg()
+    n = C.c_size_t()
+    assert lib.mi_moe_workspace_size(C.byref(c), 32, C.byref(n)) == 0 and n.value > 0
+    assert lib.mi_moe_workspace_size(C.byref(c), -1, C.byref(n)) != 0
+    assert lib.mi_moe_workspace_size(None, 1, C.byref(n)) != 0
+    h = C.c_void_p()
+    assert lib.mi_moe_create(C.byref(c), None, C.byref(h)) != 0 and "weights" in m.capi.last_error()
+    w = m.capi.Weights()                          # all NULL
+    assert lib.mi_moe_create(C.byref(c), C.byref(w), C.byref(h)) != 0 and not h.value
+    assert lib.mi_moe_forward(None, None, 1, None, None, 0, None, None) != 0
+    assert lib.mi_moe_forward(None, None, -1, None, None, 0, None, None) != 0
+    assert lib.mi_moe_destroy(None) == 0
+    # stage level
+    assert lib.mi_moe_route(None, None, None, 4, 256, 8, 2, 0, None, None, None, None, 0, None) != 0
+    assert lib.mi_moe_route(None, None, None, 4, 250, 8, 2, 0, None, None, None, None, 0, None) != 0
+    assert "hidden" in m.capi.last_error()
+    assert lib.mi_moe_dispatch(None, 8, 4, None, None, None, None, None, 0, None) != 0
+    assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 64, 64, 3, 0, 64, 4, 0,
+                                 None, None, 0, None) != 0
+    assert "transpose" in m.capi.last_error()
+    assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 64, 64, 3, 1, 64, 5, 0,
+                                 None, None, 0, None) != 0
+    assert "bits" in m.capi.last_error()
+    assert lib.mi_moe_combine(None, None, None, 4, 2, 64, None, None) != 0
+    assert lib.mi_moe_swiglu(None, None, 8, None, None) != 0
+    assert lib.mi_moe_quantize(None, 2, 100, 64, 4, None, None, None, None) != 0
+    assert "divisible" in m.capi.last_error()
+    assert lib.mi_moe_dequantize(None, None, None, 2, 128, 64, 3, None, None) != 0
+    # empty inputs succeed without touching memory
+    assert lib.mi_moe_swiglu(None, None, 0, None, None) == 0
+    assert lib.mi_moe_combine(None, None, None, 0, 2, 64, None, None) == 0
+
+
+def test_error_handler_receives_the_message(lib):
+    import mlx_rs_amd as m
+    seen = []
+    cb = m.capi.ERROR_HANDLER(lambda msg, data: seen.append(msg.decode()))
+    lib.mi_moe_set_error_handler(cb, None, C.cast(None, m.capi.ERROR_DTOR))
+    try:
+        assert lib.mi_moe_workspace_size(None, 1, None) != 0
+        assert seen and "NULL" in seen[-1]
+    finally:
+        lib.mi_moe_set_error_handler(C.cast(None, m.capi.ERROR_HANDLER), None, C.cast(None, m.capi.ERROR_DTOR))
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    import mlx_rs_amd as m
+    monkeypatch.setattr(m.capi, "_lib", None)
+    monkeypatch.setattr(m.capi, "_SO", "/nonexistent/libmi_moe.so")
+    with pytest.raises(m.MoeError):
+        m.capi.load_library()

@@ -1,0 +1,158 @@
+"""GPU parity of the stage-level entry points (through the C ABI) against the oracle: integer
+results bit-exact, floats within max-abs 2e-2 and relative Frobenius 1e-2 (bf16)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (assert_close_bf16, bits_u16, bits_u32, bf16_tensor, i32_tensor, f32_of_bits)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def m():
+    import mlx_rs_amd
+    mlx_rs_amd.load_library()
+    return mlx_rs_amd
+
+
+@pytest.mark.parametrize("T,H,E,k,mode,bias", [
+    (1, 2048, 128, 8, 0, False), (33, 2048, 128, 8, 0, True), (300, 512, 60, 6, 1, False),
+    (65, 4096, 8, 2, 2, False), (17, 256, 300, 8, 0, True), (5, 128, 5, 5, 2, False),
+])
+def test_route_bit_exact(orc, m, T, H, E, k, mode, bias):
+    print(f"route T={T} H={H} E={E} k={k} mode={mode}", flush=True)
+    rng = np.random.default_rng(T + E)
+    x = orc.f32_to_bf16(rng.normal(0, 1, (T, H)).astype(np.float32))
+    w = orc.f32_to_bf16(rng.normal(0, 0.02, (E, H)).astype(np.float32))
+    b = rng.normal(0, 1, E).astype(np.float32) if bias else None
+    cfg = orc.make_config(H, E, k, 64, 4, 64, mode)
+    inds, sc = orc.route(cfg, w, b, x)
+    gi, gs, gl = m.ops.route(bf16_tensor(x, "cuda"), bf16_tensor(w, "cuda"), k, mode,
+                             None if b is None else torch.from_numpy(b).cuda(), return_logits=True)
+    assert np.array_equal(bits_u16(gl), orc.router_logits(x, w, b)), "logits"
+    assert np.array_equal(bits_u32(gi), inds), "top-k indices"
+    assert np.array_equal(bits_u16(gs), sc), "scores"
+
+
+def test_route_ties_go_to_the_lower_expert(orc, m):
+    # identical router rows give identical logits: ties everywhere
+    H, E, k = 128, 16, 4
+    rng = np.random.default_rng(0)
+    row = orc.f32_to_bf16(rng.normal(0, 0.02, (1, H)).astype(np.float32))
+    w = np.repeat(row, E, 0)
+    x = orc.f32_to_bf16(rng.normal(0, 1, (7, H)).astype(np.float32))
+    gi, _ = m.ops.route(bf16_tensor(x, "cuda"), bf16_tensor(w, "cuda"), k, 0)
+    assert (bits_u32(gi) == np.arange(k)).all()
+    # zero activations: all logits +0
+    gi, gs = m.ops.route(bf16_tensor(np.zeros((3, H), np.uint16), "cuda"), bf16_tensor(w, "cuda"), k, 2)
+    assert (bits_u32(gi) == np.arange(k)).all()
+    assert np.array_equal(bits_u16(gs), orc.f32_to_bf16(np.full((3, k), 0.25, np.float32)))
+
+
+@pytest.mark.parametrize("P,E", [(1, 8), (8, 128), (256, 128), (4096, 8), (4097, 128), (40000, 64), (70000, 500)])
+def test_dispatch_bit_exact(orc, m, P, E):
+    print(f"dispatch P={P} E={E}", flush=True)
+    rng = np.random.default_rng(P)
+    zipf = rng.zipf(1.3, P) % E if P > 1000 else rng.integers(0, E, P)
+    flat = zipf.astype(np.uint32)
+    counts, offsets, perm, inv = orc.dispatch(flat, E)
+    g = m.ops.dispatch(i32_tensor(flat, "cuda"), E)
+    for got, ref, name in zip(g, (counts, offsets, perm, inv), ("counts", "offsets", "perm", "inv_perm")):
+        assert np.array_equal(bits_u32(got), ref), name
+    assert np.array_equal(perm, np.argsort(flat, kind="stable"))
+
+
+@pytest.mark.parametrize("bits,M,N,K,E,n_idx,xb", [
+    (4, 32, 64, 128, 3, 2, 5),      # the reference's test shapes (K raised to a multiple of 128 for 4-bit)
+    (8, 32, 64, 64, 3, 2, 1),       # ... and its exact shapes with 8-bit codes
+    (4, 1, 768, 2048, 16, 40, 40), (8, 1, 256, 512, 4, 300, 300), (4, 3, 48, 256, 5, 7, 4),
+])
+def test_gather_qmm_matches_oracle(orc, m, bits, M, N, K, E, n_idx, xb):
+    print(f"gather_qmm bits={bits} M={M} N={N} K={K} E={E} n_idx={n_idx}", flush=True)
+    rng = np.random.default_rng(N + K)
+    w = rng.normal(0, 0.02, (E * N, K)).astype(np.float32)   # outputs stay below 4: one bf16 ulp < 2e-2
+    q, s, b = orc.quantize(w, bits, 64)
+    q, s, b = q.reshape(E, N, -1), s.reshape(E, N, -1), b.reshape(E, N, -1)
+    x = orc.f32_to_bf16(rng.normal(0, 1, (xb, M, K)).astype(np.float32))
+    rhs = rng.integers(0, E, n_idx).astype(np.uint32)
+    lhs = None if xb == n_idx else rng.integers(0, xb, n_idx).astype(np.uint32)
+    ref = orc.gather_qmm(x, q, s, b, lhs, rhs, bits, want="bf16")
+    got = m.ops.gather_qmm(bf16_tensor(x, "cuda"), i32_tensor(q, "cuda"), bf16_tensor(s, "cuda"),
+                           bf16_tensor(b, "cuda"), None if lhs is None else i32_tensor(lhs, "cuda"),
+                           i32_tensor(rhs, "cuda"), True, 64, bits, sorted_indices=False)
+    assert_close_bf16(bits_u16(got), ref, what="gather_qmm")
+    # the sorted hint changes nothing (test_gather_mm_sorted, ops/arithmetic.rs:3214-3238)
+    o = np.argsort(rhs, kind="stable")
+    got2 = m.ops.gather_qmm(bf16_tensor(x, "cuda"), i32_tensor(q, "cuda"), bf16_tensor(s, "cuda"),
+                            bf16_tensor(b, "cuda"), i32_tensor((np.arange(n_idx) if lhs is None else lhs)[o].astype(np.uint32), "cuda"),
+                            i32_tensor(rhs[o], "cuda"), True, 64, bits, sorted_indices=True)
+    assert np.array_equal(bits_u16(got2), bits_u16(got)[o])
+
+
+def test_gather_qmm_unit_scale_is_exact(orc, m):
+    rng = np.random.default_rng(9)
+    E, N, K = 2, 16, 256
+    codes = rng.integers(0, 16, (E, N, K)).astype(np.uint32)
+    q = np.zeros((E, N, K // 8), np.uint32)
+    for j in range(8):
+        q |= codes[..., j::8] << np.uint32(4 * j)
+    one = orc.f32_to_bf16(np.ones((E, N, K // 64), np.float32))
+    zero = np.zeros((E, N, K // 64), np.uint16)
+    xi = np.zeros((5, 1, K), np.int64)   # 8 entries of +-1 per row: |sum| <= 120, exact in bf16
+    for j in range(5):
+        xi[j, 0, rng.choice(K, 8, replace=False)] = rng.choice([-1, 1], 8)
+    got = m.ops.gather_qmm(bf16_tensor(orc.f32_to_bf16(xi.astype(np.float32)), "cuda"), i32_tensor(q, "cuda"),
+                           bf16_tensor(one, "cuda"), bf16_tensor(zero, "cuda"), None,
+                           i32_tensor(np.array([1, 0, 1, 1, 0], np.uint32), "cuda"))
+    ref = np.stack([xi[j, 0] @ codes[e].astype(np.int64).T for j, e in enumerate([1, 0, 1, 1, 0])])
+    assert np.array_equal(f32_of_bits(bits_u16(got))[:, 0].astype(np.int64), ref)  # |sum| < 256: exact in bf16
+
+
+def test_swiglu_and_combine(orc, m):
+    rng = np.random.default_rng(3)
+    # |gate|, |up| <= 1.9: |silu(gate) * up| < 4, so one bf16 ulp stays below the 2e-2 bound
+    g = orc.f32_to_bf16(np.clip(rng.normal(0, 0.9, (77, 96)), -1.9, 1.9).astype(np.float32))
+    u = orc.f32_to_bf16(np.clip(rng.normal(0, 0.9, (77, 96)), -1.9, 1.9).astype(np.float32))
+    got = m.ops.swiglu(bf16_tensor(g, "cuda"), bf16_tensor(u, "cuda"))
+    assert_close_bf16(bits_u16(got), orc.swiglu_bf16(g, u), what="swiglu vs op-by-op oracle")
+    assert_close_bf16(bits_u16(got), orc.swiglu_f32(f32_of_bits(g), f32_of_bits(u)), max_abs=2e-2, rel_fro=3e-3,
+                      what="swiglu vs single-rounding oracle")
+    T, k, H = 50, 8, 2048
+    y = orc.f32_to_bf16(rng.normal(0, 1, (T * k, H)).astype(np.float32))
+    sc = orc.f32_to_bf16(rng.uniform(0, 0.3, (T, k)).astype(np.float32))
+    inv = rng.permutation(T * k).astype(np.uint32)
+    for ip in (inv, None):
+        got = m.ops.combine(bf16_tensor(y, "cuda"), bf16_tensor(sc, "cuda"), None if ip is None else i32_tensor(ip, "cuda"))
+        assert np.array_equal(bits_u16(got), orc.combine(y, sc, ip)), "combine is a fixed-order fp32 sum: bit-exact"
+
+
+@pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (2, 64), (4, 32), (8, 128)])
+def test_quantize_dequantize_bit_exact(orc, m, bits, group):
+    rng = np.random.default_rng(bits + group)
+    w = rng.normal(0, 0.02, (96, 4 * group)).astype(np.float32)
+    w[3] = 0.0
+    w[4] = 0.25
+    q, s, b = orc.quantize(w, bits, group)
+    gq, gs, gb = m.ops.quantize(torch.from_numpy(w).cuda(), group, bits)
+    assert np.array_equal(bits_u32(gq), q) and np.array_equal(bits_u16(gs), s) and np.array_equal(bits_u16(gb), b)
+    wh = m.ops.dequantize(gq, gs, gb, group, bits).cpu().numpy()
+    assert np.array_equal(wh, orc.dequantize(q, s, b, bits, group))
+    # the reference's known-answer case (ops/quantization.rs:298-315) on the device
+    x = np.tile(np.arange(512, dtype=np.float32), (128, 1))
+    gq, gs, gb = m.ops.quantize(torch.from_numpy(x).cuda(), 128, bits)
+    assert tuple(gq.shape) == (128, 512 * bits // 32) and tuple(gs.shape) == (128, 4)
+    xh = m.ops.dequantize(gq, gs, gb, 128, bits).cpu().numpy()
+    assert np.abs(x - xh).max() <= 127.0 / (1 << bits) + 2.0   # + bf16 rounding of a bias near 511
+
+
+def test_errors_reach_the_caller(m):
+    x = torch.zeros((4, 100), dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros((8, 100), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(m.MoeError, match="hidden"):
+        m.ops.route(x, w, 2)
+    with pytest.raises(m.MoeError, match="divisible"):
+        m.ops.quantize(torch.zeros((4, 100), device="cuda"), 64, 4)
+    with pytest.raises(m.MoeError, match="top_k"):
+        m.ops.route(torch.zeros((4, 128), dtype=torch.bfloat16, device="cuda"),
+                    torch.zeros((8, 128), dtype=torch.bfloat16, device="cuda"), 9)

@@ -102,7 +102,8 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.offsets = cv.take<uint32_t>(c.n_experts + 1);
   f.work = cv.take<uint32_t>((size_t)c.n_experts * 16);
   // M tiles of the tiled kernel: at most one partial tile per long segment plus P / tile full ones
-  f.max_mtiles = P >= kBigThreshold ? (int)(P / kBigTileM + (P / kBigThreshold < c.n_experts ? P / kBigThreshold : c.n_experts)) : 0;
+  // (a segment is at most T rows long: no token picks an expert twice)
+  f.max_mtiles = T >= kBigThreshold ? (int)(P / kBigTileM + (P / kBigThreshold < c.n_experts ? P / kBigThreshold : c.n_experts)) : 0;
   f.mtiles = cv.take<uint32_t>(4 + (size_t)f.max_mtiles * 4);
   f.perm = cv.take<uint32_t>((size_t)P);
   f.inv_perm = cv.take<uint32_t>((size_t)P);

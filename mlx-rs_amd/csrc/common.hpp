@@ -7,7 +7,7 @@
 namespace mi_moe {
 
 constexpr int kWave = 64;
-constexpr int kBigThreshold = 24;  // segments with at least this many rows use the tiled kernel
+constexpr int kBigThreshold = 48;  // segments with at least this many rows use the tiled kernel
 constexpr int kBigTileM = 256;     // rows per M tile of the tiled kernel
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;

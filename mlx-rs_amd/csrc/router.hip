@@ -87,6 +87,84 @@ __global__ __launch_bounds__(256) void router_logits_kernel(
     }
 }
 
+// Prefill-sized T: the same fp64 accumulation on the matrix cores (v_mfma_f64_16x16x4_f64).
+// A block computes a 32-token x 32-expert tile; its 4 waves split H in 32-wide chunks and the
+// partial tiles are added in wave order through LDS.  Lane (i = lane & 15, kq = lane >> 4)
+// loads 8 consecutive h of row i per chunk; MFMA step s multiplies element s of every lane, so
+// the four kq lanes of a row cover 32 consecutive h in 8 steps (any K order gives the same sum).
+typedef __attribute__((__vector_size__(4 * sizeof(double)))) double f64x4_t;
+
+__global__ __launch_bounds__(256) void router_logits_mfma_kernel(
+    const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg,
+    const float *__restrict__ bias, int64_t T, int H, int E, uint16_t *__restrict__ logits) {
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = lane & 15, kq = lane >> 4;
+  const int64_t t0 = (int64_t)blockIdx.x * 32;
+  const int e0 = blockIdx.y * 32;
+  const uint16_t *xr[2], *wr[2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    const int64_t t = t0 + 16 * a + i;
+    const int e = e0 + 16 * a + i;
+    xr[a] = x + (t < T ? t : T - 1) * H + kq * 8;
+    wr[a] = wg + (int64_t)(e < E ? e : E - 1) * H + kq * 8;
+  }
+  f64x4_t acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) acc[a][b] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+
+  for (int c = wave; c < H / 32; c += 4) {
+    uint32_t xa[2][4], wb[2][4];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const uint4 v = *reinterpret_cast<const uint4 *>(xr[a] + c * 32);
+      const uint4 u = *reinterpret_cast<const uint4 *>(wr[a] + c * 32);
+      xa[a][0] = v.x; xa[a][1] = v.y; xa[a][2] = v.z; xa[a][3] = v.w;
+      wb[a][0] = u.x; wb[a][1] = u.y; wb[a][2] = u.z; wb[a][3] = u.w;
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      double av[2], bv[2];
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        av[a] = (double)((s & 1) ? bf16hi_to_f32(xa[a][s >> 1]) : bf16lo_to_f32(xa[a][s >> 1]));
+        bv[a] = (double)((s & 1) ? bf16hi_to_f32(wb[a][s >> 1]) : bf16lo_to_f32(wb[a][s >> 1]));
+      }
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[a], bv[b], acc[a][b], 0, 0, 0);
+    }
+  }
+
+  __shared__ double part[4][4][4][64];  // [wave][tile][r][lane]
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) part[wave][a * 2 + b][r][lane] = acc[a][b][r];
+  __syncthreads();
+  // wave w finishes tile w = (a, b) = (w >> 1, w & 1); a lane's register r holds D[4 r + kq][i]
+  // (fp64 tiles interleave the rows over the four lane groups, unlike the fp32 16x16 layout)
+  const int a = wave >> 1, b = wave & 1;
+  const int e = e0 + 16 * b + i;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    double s = ((part[0][wave][r][lane] + part[1][wave][r][lane]) + part[2][wave][r][lane]) +
+               part[3][wave][r][lane];
+    const int64_t t = t0 + 16 * a + 4 * r + kq;
+    if (t < T && e < E) {
+      if (bias) s += (double)bias[e];
+      logits[t * E + e] = f32_to_bf16((float)s);
+    }
+  }
+}
+
 hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,
                                 int64_t T, int H, int E, uint16_t *logits, hipStream_t st) {
   if (T == 0) return hipSuccess;
@@ -94,8 +172,8 @@ hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const flo
     dim3 grid((unsigned)T, (unsigned)((E + 3) / 4));
     router_logits_kernel<1, 1><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
   } else {
-    dim3 grid((unsigned)((T + 3) / 4), (unsigned)((E + 15) / 16));
-    router_logits_kernel<4, 4><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+    dim3 grid((unsigned)((T + 31) / 32), (unsigned)((E + 31) / 32));
+    router_logits_mfma_kernel<<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
   }
   return hipGetLastError();
 }

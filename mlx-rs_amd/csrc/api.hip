@@ -87,7 +87,7 @@ struct ForwardWs {
   uint32_t *counts, *offsets, *work, *mtiles, *perm, *inv_perm, *src_of;
   int max_mtiles;
   void *disp_scratch;
-  uint16_t *hh, *y;
+  uint16_t *hh, *y, *xperm;
   size_t bytes;
 };
 
@@ -111,6 +111,7 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.disp_scratch = cv.take<char>(dispatch_workspace_bytes(c.n_experts, P));
   f.hh = cv.take<uint16_t>((size_t)P * c.intermediate);
   f.y = cv.take<uint16_t>((size_t)P * c.hidden);
+  f.xperm = cv.take<uint16_t>(f.max_mtiles && c.bits == 4 ? (size_t)T * c.hidden : 0);
   f.bytes = cv.off;
   return f;
 }
@@ -207,8 +208,15 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   a.bits = c.bits;
   a.total_rows = P;
   a.max_rows_per_expert = T;  // a token picks an expert at most once
+  // 4-bit: the tiled kernel reads activations with paired 8-blocks; h is produced that way,
+  // x is copied once per forward (prefill-sized T only)
+  const bool paired = c.bits == 4;
+  if (f.max_mtiles && paired) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
   // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
   a.x = x;
+  a.x_perm = paired ? (f.max_mtiles ? f.xperm : nullptr) : x;
+  a.x_paired = false;
+  a.y_paired = paired;
   a.src_rows = f.src_of;
   a.src_in_work = true;
   a.dst_rows = nullptr;
@@ -221,6 +229,9 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   MI_STAGE_DONE();
   // down: rows read in sorted order, written back in (token, slot) order
   a.x = f.hh;
+  a.x_perm = f.hh;
+  a.x_paired = paired;
+  a.y_paired = false;
   a.src_rows = nullptr;
   a.src_in_work = false;
   a.dst_rows = f.perm;

@@ -89,6 +89,10 @@ __device__ __forceinline__ float wave_max_f32(float v) {
 // Each returns hipSuccess or the launch error.  All pointers are device pointers.
 struct GroupedArgs {
   const uint16_t *x;        // bf16 rows of length K
+  const uint16_t *x_perm;   // the same rows in the order the tiled kernel reads (4-bit: 8-blocks paired
+                            // as x0,x4,x1,x5,x2,x6,x3,x7; 8-bit: identical to x)
+  bool x_paired;            // x itself is already in the paired order
+  bool y_paired;            // write the output columns in the paired order
   const uint32_t *src_rows; // x row of sorted row r, or nullptr = r
   bool src_in_work;         // the records' inline source rows equal src_rows (saves a dependent load)
   const uint32_t *dst_rows; // output row of sorted row r, or nullptr = r
@@ -115,6 +119,7 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
                            void *scratch, hipStream_t st);
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
+hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *out, hipStream_t st);
 hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
                            uint32_t *work, hipStream_t st);

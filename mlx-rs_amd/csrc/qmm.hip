@@ -258,7 +258,7 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
           sum += __shfl_xor(sum, 4, kWave);
           if (blk < K / 8) {
             uint4 p = w;
-            if constexpr (BITS == 4) {
+            if (BITS == 4 && !a.x_paired) {
               p.x = (w.x & 0xffffu) | (w.z << 16);
               p.y = (w.x >> 16) | (w.z & 0xffff0000u);
               p.z = (w.y & 0xffffu) | (w.w << 16);
@@ -402,7 +402,9 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
           float v;
           if constexpr (GLU) v = silu_mul(res[0][r], res[1][r]);
           else v = res[0][r];
-          a.y[dst * N + n] = (uint16_t)(cvt_pk_bf16(v, 0.f) & 0xffffu);
+          int col = n;
+          if (a.y_paired) col = (n & ~7) | ((n & 7) < 4 ? 2 * (n & 7) : 2 * ((n & 7) - 4) + 1);
+          a.y[dst * N + col] = (uint16_t)(cvt_pk_bf16(v, 0.f) & 0xffffu);
         }
       }
     }

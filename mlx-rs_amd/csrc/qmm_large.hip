@@ -21,28 +21,32 @@ namespace mi_moe {
 namespace {
 
 constexpr int BM = kBigTileM;  // token rows per block
-constexpr int BK = 64;         // one quantisation group per K step
+constexpr int BK = 32;         // K step (two steps per quantisation group)
 constexpr int BR = 128;        // weight rows per block (GLU: 64 gate + 64 up)
-constexpr int LDK = 72;        // LDS row stride in bf16 (144 bytes: conflict-free 16-byte reads)
 
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
 
-__device__ __forceinline__ f32x16_t mfma32(const uint4 &a, const uint4 &b, f32x16_t c) {
-  const u32x4_t av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                 __builtin_bit_cast(bf16x8_t, bv), c, 0, 0, 0);
+__device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
+
+// LDS tiles hold rows of 32 bf16 (four 16-byte chunks) at a stride of 80 bytes: consecutive
+// rows reading the same chunk start 20 banks apart, which keeps 16-byte reads of 8 or 16
+// consecutive rows free of bank conflicts (measured: SQ_LDS_BANK_CONFLICT = 0).
+constexpr int LDR = 5;  // row stride in uint4 units
+__device__ __forceinline__ int tile_off(int row, int chunk) { return row * LDR + chunk; }
 
 }  // namespace
 
 template <int BITS, bool GLU>
-__global__ __launch_bounds__(256, 2) void qmm_large_kernel(GroupedArgs a, int n_ntiles) {
-  constexpr int NI = GLU ? 64 : 128;          // distinct output columns per block
-  constexpr int BQ = BITS == 4 ? 1 : 2;       // 16-byte weight loads per thread per K step
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qmm_large_kernel(GroupedArgs a, int n_ntiles) {
+  constexpr int NI = GLU ? 64 : 128;  // distinct output columns per block
 
   // block -> (M tile, N tile): blocks of one M tile share the gathered token rows, so they
   // are given consecutive ids on ONE XCD (ids are dealt round-robin over the 8 XCDs)
@@ -63,92 +67,91 @@ __global__ __launch_bounds__(256, 2) void qmm_large_kernel(GroupedArgs a, int n_
   const int n0 = nt * NI;
   const int row_bytes = K * BITS / 8, gpr = K / 64;
 
-  __shared__ __align__(16) uint16_t As[BM * LDK];
-  __shared__ __align__(16) uint16_t Bs[BR * LDK];
+  __shared__ u32x4_t As[2][BM * LDR];
+  __shared__ u32x4_t Bs[2][BR * LDR];
 
   // ---- global -> register stage
-  // A: thread covers 8 rows (rg + 32 j) x one 8-element piece (cp) of the K step
-  const int cp = tid & 7, rg = tid >> 3;
-  const uint16_t *arow[8];
-#pragma unroll
-  for (int jj = 0; jj < 8; ++jj) {
-    int tr = rg + 32 * jj;
+  // A: the activations arrive with every 8-block already in the (x0,x4,x1,x5,x2,x6,x3,x7) order
+  // of the nibble unpacking (4-bit), so a row chunk is copied as it is.  Thread: chunk acp of
+  // rows arg + 64 j.
+  const int acp = tid & 3, arg = tid >> 2;
+  auto a_row_ptr = [&](int tr) {
     tr = tr < rows ? tr : rows - 1;  // rows past the segment repeat its last row (never stored)
     const int64_t r = row0 + tr;
     const int64_t src = a.src_rows ? (int64_t)a.src_rows[r] : r;
-    arow[jj] = a.x + src * K + cp * 8;
-  }
-  // B: thread covers half a K step (32 codes) of weight row br
+    return a.x_perm + src * K + acp * 8;
+  };
+  const uint16_t *const arow[4] = {a_row_ptr(arg), a_row_ptr(arg + 64), a_row_ptr(arg + 128), a_row_ptr(arg + 192)};
+  // B: thread covers 16 codes (half a K step) of weight row br; waves 0,1 / 2,3 hold gate / up
   const int br = tid >> 1, bh = tid & 1;
-  const int mat = GLU ? (br >> 6) : 0;
+  const int mat = GLU ? (wave >> 1) : 0;  // wave-uniform
   const int nrow = GLU ? n0 + (br & 63) : n0 + br;  // rows >= N read zeros through the descriptor
   const int64_t ebase = (int64_t)e * N;
-  const uint32_t *wbase = (mat ? a.w1 : a.w0) + ebase * (row_bytes / 4);
-  const uint16_t *sbase = (mat ? a.s1 : a.s0) + ebase * gpr;
-  const uint16_t *bbase = (mat ? a.b1 : a.b0) + ebase * gpr;
-  const __amdgpu_buffer_rsrc_t wr = make_rsrc(wbase, (uint32_t)N * row_bytes);
-  const __amdgpu_buffer_rsrc_t sr = make_rsrc(sbase, (uint32_t)N * gpr * 2);
-  const __amdgpu_buffer_rsrc_t brs = make_rsrc(bbase, (uint32_t)N * gpr * 2);
-  const uint32_t w_voff = (uint32_t)nrow * row_bytes + bh * (BITS == 4 ? 16 : 32);
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc((mat ? a.w1 : a.w0) + ebase * (row_bytes / 4), (uint32_t)N * row_bytes);
+  const __amdgpu_buffer_rsrc_t sr = make_rsrc((mat ? a.s1 : a.s0) + ebase * gpr, (uint32_t)N * gpr * 2);
+  const __amdgpu_buffer_rsrc_t brs = make_rsrc((mat ? a.b1 : a.b0) + ebase * gpr, (uint32_t)N * gpr * 2);
+  const uint32_t w_voff = (uint32_t)nrow * row_bytes + bh * (BITS == 4 ? 8 : 16);
   const uint32_t g_voff = (uint32_t)nrow * gpr * 2;
 
-  uint4 areg[8];
-  u32x4_t breg[BQ];
-  uint32_t sreg, bireg;
-  auto gload = [&](int ks) {
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) areg[jj] = *reinterpret_cast<const uint4 *>(arow[jj] + ks * BK);
-#pragma unroll
-    for (int q = 0; q < BQ; ++q)
-      breg[q] = __builtin_amdgcn_raw_buffer_load_b128(wr, w_voff + q * 16, ks * (BK * BITS / 8), 0);
-    sreg = __builtin_amdgcn_raw_buffer_load_b16(sr, g_voff, ks * 2, 0);
-    bireg = __builtin_amdgcn_raw_buffer_load_b16(brs, g_voff, ks * 2, 0);
+  // Two sets of staging registers (plain scalars: they must not end up in scratch or LDS), so
+  // that global loads are issued two K steps before their data is needed.
+  struct Stage {
+    u32x4_t a0, a1, a2, a3;
+    uint32_t b0w, b1w, b2w, b3w;  // 4-bit: two words used
+    uint32_t sreg, bireg;
+  };
+  auto gload = [&](int ks, Stage &R) __attribute__((always_inline)) {
+    R.a0 = *reinterpret_cast<const u32x4_t *>(arow[0] + ks * BK);
+    R.a1 = *reinterpret_cast<const u32x4_t *>(arow[1] + ks * BK);
+    R.a2 = *reinterpret_cast<const u32x4_t *>(arow[2] + ks * BK);
+    R.a3 = *reinterpret_cast<const u32x4_t *>(arow[3] + ks * BK);
+    if constexpr (BITS == 4) {
+      const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(wr, w_voff, ks * 16, 0);
+      R.b0w = v[0];
+      R.b1w = v[1];
+    } else {
+      const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(wr, w_voff, ks * 32, 0);
+      R.b0w = v[0];
+      R.b1w = v[1];
+      R.b2w = v[2];
+      R.b3w = v[3];
+    }
+    R.sreg = __builtin_amdgcn_raw_buffer_load_b16(sr, g_voff, (ks >> 1) * 2, 0);
+    R.bireg = __builtin_amdgcn_raw_buffer_load_b16(brs, g_voff, (ks >> 1) * 2, 0);
   };
 
-  // ---- register -> LDS stage
-  auto stage = [&]() {
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-      uint4 v = areg[jj];
-      if constexpr (BITS == 4) {  // pair (x_i, x_{i+4}) like the nibble unpacking below
-        uint4 p;
-        p.x = (v.x & 0xffffu) | (v.z << 16);
-        p.y = (v.x >> 16) | (v.z & 0xffff0000u);
-        p.z = (v.y & 0xffffu) | (v.w << 16);
-        p.w = (v.y >> 16) | (v.w & 0xffff0000u);
-        v = p;
-      }
-      *reinterpret_cast<uint4 *>(&As[(rg + 32 * jj) * LDK + cp * 8]) = v;
-    }
-    const float sc = bf16lo_to_f32(sreg);
-    float bi = bf16lo_to_f32(bireg);
-    uint16_t *bdst = &Bs[br * LDK + bh * 32];
+  // ---- register -> LDS stage: copy A, dequantise B once for the whole block
+  auto stage = [&](int buf, const Stage &R) __attribute__((always_inline)) {
+    As[buf][tile_off(arg, acp)] = R.a0;
+    As[buf][tile_off(arg + 64, acp)] = R.a1;
+    As[buf][tile_off(arg + 128, acp)] = R.a2;
+    As[buf][tile_off(arg + 192, acp)] = R.a3;
+    const float sc = bf16lo_to_f32(R.sreg);
+    float bi = bf16lo_to_f32(R.bireg);
     if constexpr (BITS == 4) {
       bi = __builtin_fmaf(-128.0f, sc, bi);  // codes are expanded as 128 + q
 #pragma unroll
-      for (int wi = 0; wi < 4; ++wi) {
-        const uint32_t w = breg[0][wi];
+      for (int wi = 0; wi < 2; ++wi) {
+        const uint32_t w = wi == 0 ? R.b0w : R.b1w;
         uint32_t o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t pr = ((w >> (4 * i)) & 0x000f000fu) | 0x43004300u;  // (128+q_i, 128+q_{i+4})
           o[i] = cvt_pk_bf16(__builtin_fmaf(sc, bf16lo_to_f32(pr), bi), __builtin_fmaf(sc, bf16hi_to_f32(pr), bi));
         }
-        *reinterpret_cast<uint4 *>(bdst + wi * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+        Bs[buf][tile_off(br, 2 * bh + wi)] = u32x4_t{o[0], o[1], o[2], o[3]};
       }
     } else {
 #pragma unroll
-      for (int q = 0; q < BQ; ++q)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {  // 8 codes = two words -> one 16-byte LDS store
-          const uint32_t wA = breg[q][2 * h], wB = breg[q][2 * h + 1];
-          uint32_t o[4];
-          o[0] = cvt_pk_bf16(__builtin_fmaf(sc, (float)(wA & 0xffu), bi), __builtin_fmaf(sc, (float)((wA >> 8) & 0xffu), bi));
-          o[1] = cvt_pk_bf16(__builtin_fmaf(sc, (float)((wA >> 16) & 0xffu), bi), __builtin_fmaf(sc, (float)(wA >> 24), bi));
-          o[2] = cvt_pk_bf16(__builtin_fmaf(sc, (float)(wB & 0xffu), bi), __builtin_fmaf(sc, (float)((wB >> 8) & 0xffu), bi));
-          o[3] = cvt_pk_bf16(__builtin_fmaf(sc, (float)((wB >> 16) & 0xffu), bi), __builtin_fmaf(sc, (float)(wB >> 24), bi));
-          *reinterpret_cast<uint4 *>(bdst + q * 16 + h * 8) = make_uint4(o[0], o[1], o[2], o[3]);
-        }
+      for (int h = 0; h < 2; ++h) {  // 8 codes = two words -> one chunk
+        const uint32_t wA = h == 0 ? R.b0w : R.b2w, wB = h == 0 ? R.b1w : R.b3w;
+        uint32_t o[4];
+        o[0] = cvt_pk_bf16(__builtin_fmaf(sc, (float)(wA & 0xffu), bi), __builtin_fmaf(sc, (float)((wA >> 8) & 0xffu), bi));
+        o[1] = cvt_pk_bf16(__builtin_fmaf(sc, (float)((wA >> 16) & 0xffu), bi), __builtin_fmaf(sc, (float)(wA >> 24), bi));
+        o[2] = cvt_pk_bf16(__builtin_fmaf(sc, (float)(wB & 0xffu), bi), __builtin_fmaf(sc, (float)((wB >> 8) & 0xffu), bi));
+        o[3] = cvt_pk_bf16(__builtin_fmaf(sc, (float)((wB >> 16) & 0xffu), bi), __builtin_fmaf(sc, (float)(wB >> 24), bi));
+        Bs[buf][tile_off(br, 2 * bh + h)] = u32x4_t{o[0], o[1], o[2], o[3]};
+      }
     }
   };
 
@@ -161,33 +164,53 @@ __global__ __launch_bounds__(256, 2) void qmm_large_kernel(GroupedArgs a, int n_
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[m][s][r] = 0.f;
   const int ln = lane & 31, kb = lane >> 5;
-  const int brow0 = GLU ? 32 * wn : 64 * wn;       // first sub-tile: gate rows / first 32 rows
-  const int brow1 = GLU ? 64 + 32 * wn : 64 * wn + 32;  // second: the matching up rows / next 32
-  const uint16_t *ap = &As[(128 * wm + ln) * LDK + kb * 32];
-  const uint16_t *bp0 = &Bs[(brow0 + ln) * LDK + kb * 32];
-  const uint16_t *bp1 = &Bs[(brow1 + ln) * LDK + kb * 32];
+  const int brow0 = (GLU ? 32 * wn : 64 * wn) + ln;            // gate rows / first 32 rows
+  const int brow1 = (GLU ? 64 + 32 * wn : 64 * wn + 32) + ln;  // the matching up rows / next 32
+  const int arow0 = 128 * wm + ln;
 
-  const int nk = K / BK;
-  gload(0);
-  for (int ks = 0; ks < nk; ++ks) {
-    __syncthreads();  // every wave has finished reading the previous K step
-    stage();
-    __syncthreads();
-    if (ks + 1 < nk) gload(ks + 1);
+  auto mma = [&](int cur) __attribute__((always_inline)) {
 #pragma unroll
-    for (int ss = 0; ss < 4; ++ss) {
-      const uint4 b0 = *reinterpret_cast<const uint4 *>(bp0 + ss * 8);
-      const uint4 b1 = *reinterpret_cast<const uint4 *>(bp1 + ss * 8);
+    for (int ss = 0; ss < 2; ++ss) {
+      const int c = 2 * kb + ss;
+      const u32x4_t b0 = Bs[cur][tile_off(brow0, c)];
+      const u32x4_t b1 = Bs[cur][tile_off(brow1, c)];
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        const uint4 av = *reinterpret_cast<const uint4 *>(ap + m * 32 * LDK + ss * 8);
+        const u32x4_t av = As[cur][tile_off(arow0 + 32 * m, c)];
         acc[m][0] = mfma32(av, b0, acc[m][0]);
         acc[m][1] = mfma32(av, b1, acc[m][1]);
       }
     }
+  };
+
+  // K loop, two steps per trip (nk is even: K is a multiple of 64).  Entering step ks: LDS buffer
+  // ks & 1 holds step ks, register set R1/R0 holds step ks + 1, the load of step ks + 2 is in flight.
+  const int nk = K / BK;
+  Stage R0, R1;
+  gload(0, R0);
+  gload(1, R1);
+  stage(0, R0);
+  if (nk > 2) gload(2, R0);
+  __syncthreads();
+  for (int ks = 0; ks < nk; ks += 2) {
+    stage(1, R1);                          // step ks + 1 -> buffer 1 (last read before the previous barrier)
+    if (ks + 3 < nk) gload(ks + 3, R1);
+    mma(0);                                // step ks
+    __syncthreads();
+    if (ks + 2 < nk) stage(0, R0);         // step ks + 2 -> buffer 0
+    if (ks + 4 < nk) gload(ks + 4, R0);
+    mma(1);                                // step ks + 1
+    __syncthreads();
   }
 
-  // ---- epilogue: D[i][j], lane holds column j = lane % 32 and rows 8 (r/4) + 4 (lane/32) + r%4
+  // ---- epilogue: D[i][j], lane holds column j = lane % 32 and rows 8 (r/4) + 4 (lane/32) + r%4.
+  // perm_out: columns are written in the paired order within each 8-block (what a 4-bit
+  // consumer of these rows expects as its activations).
+  auto out_col = [&](int col) {
+    if (!a.y_paired) return col;
+    const int jj = col & 7;
+    return (col & ~7) | (jj < 4 ? 2 * jj : 2 * (jj - 4) + 1);
+  };
 #pragma unroll
   for (int m = 0; m < 4; ++m)
 #pragma unroll
@@ -200,21 +223,43 @@ __global__ __launch_bounds__(256, 2) void qmm_large_kernel(GroupedArgs a, int n_
           const int col = n0 + 32 * wn + ln;
           if (col < N) {
             const float g = acc[m][0][r], u = acc[m][1][r];
-            a.y[dst * N + col] = (uint16_t)(cvt_pk_bf16(g / (1.0f + __expf(-g)) * u, 0.f) & 0xffffu);
+            a.y[dst * N + out_col(col)] = (uint16_t)(cvt_pk_bf16(g / (1.0f + __expf(-g)) * u, 0.f) & 0xffffu);
           }
         } else {
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
             const int col = n0 + 64 * wn + 32 * s + ln;
-            if (col < N) a.y[dst * N + col] = (uint16_t)(cvt_pk_bf16(acc[m][s][r], 0.f) & 0xffffu);
+            if (col < N) a.y[dst * N + out_col(col)] = (uint16_t)(cvt_pk_bf16(acc[m][s][r], 0.f) & 0xffffu);
           }
         }
       }
     }
 }
 
+// Activation rows with every 8-block reordered to (x0,x4,x1,x5,x2,x6,x3,x7): the order in which
+// one and+or per register unpacks the eight 4-bit codes of a word.
+__global__ __launch_bounds__(256) void pair_rows_kernel(const uint4 *__restrict__ x, int64_t n, uint4 *__restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const uint4 v = x[i];
+  uint4 p;
+  p.x = (v.x & 0xffffu) | (v.z << 16);
+  p.y = (v.x >> 16) | (v.z & 0xffff0000u);
+  p.z = (v.y & 0xffffu) | (v.w << 16);
+  p.w = (v.y >> 16) | (v.w & 0xffff0000u);
+  out[i] = p;
+}
+
+hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *out, hipStream_t st) {
+  const int64_t n = rows * K / 8;
+  if (n == 0) return hipSuccess;
+  pair_rows_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(reinterpret_cast<const uint4 *>(x), n,
+                                                               reinterpret_cast<uint4 *>(out));
+  return hipGetLastError();
+}
+
 hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
-  if (!a.mtiles || a.max_mtiles <= 0) return hipSuccess;
+  if (!a.mtiles || a.max_mtiles <= 0 || !a.x_perm) return hipSuccess;
   const int ni = glu ? 64 : 128;
   const int n_ntiles = (a.N + ni - 1) / ni;
   const unsigned grid = (unsigned)((a.max_mtiles + 7) / 8) * 8u * (unsigned)n_ntiles;

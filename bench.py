@@ -22,6 +22,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+# HBM bytes per launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE scaled by
+# what the same counters read for a plain copy kernel (profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt);
+# counters cannot be read from inside this script, so the figure is carried here per workload.
+MEASURED_TRAFFIC_BYTES = {"decode": 2.060e8}
 
 
 def parse():
@@ -35,6 +39,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--only-headline", action="store_true", help="run only the headline batch of the workload")
+    ap.add_argument("--copy-probe", type=int, default=0,
+                    help="first launch N plain 256 MiB copy kernels (a known-size reference for profiler counters)")
     return ap.parse_args()
 
 
@@ -75,6 +82,16 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     cfg_name, batches, headline, zipf_s, bound = WORKLOADS[args.workload]
+    if args.only_headline:
+        batches = [headline]
+    if args.copy_probe:
+        # an elementwise kernel that reads 256 MiB and writes 256 MiB
+        src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.copy_probe):
+            torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     cfg = synth.CONFIGS[cfg_name]
     per_expert = synth.layer_bytes_per_expert(cfg)
     layer_bytes = per_expert * cfg.n_experts
@@ -169,12 +186,15 @@ def main():
     if bound == "hbm":
         achieved = head["gu_bytes"] / (head["gu_ms"] * 1e-3) / 1e9
         roofline = {"kernel": "qmm_small_kernel (gate/up + SwiGLU)", "bound": "hbm", "achieved": achieved,
-                    "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None}
+                    "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "algorithmic_bytes_per_launch": head["gu_bytes"], "kernel_us": head["gu_ms"] * 1e3}
     else:
         achieved = head["gu_flops"] / (head["gu_ms"] * 1e-3) / 1e12
         roofline = {"kernel": "grouped qmm (gate/up + SwiGLU)", "bound": "mfma", "achieved": achieved,
                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                    "traffic": None}
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "algorithmic_flops_per_launch": head["gu_flops"], "kernel_us": head["gu_ms"] * 1e3}
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -428,7 +428,6 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   int kw = 1;
   if (tiles < 4096 && chunks >= 8) kw = 4;
   else if (tiles < 8192 && chunks >= 4) kw = 2;
-  if (const char *env = getenv("MI_MOE_KW")) kw = atoi(env);
   const int nw = 4 / kw;
   dim3 grid((unsigned)((a.N + 16 * nw - 1) / (16 * nw)), (unsigned)a.max_active);
   if (kw == 4) qmm_small_kernel<BITS, GLU, 4><<<grid, 256, lds, st>>>(a, tt);

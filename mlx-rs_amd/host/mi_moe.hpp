@@ -1,0 +1,359 @@
+// mi_moe.hpp -- header-only C++17 host layer over the C ABI of libmi_moe (include/mi_moe.h).
+//
+// It mirrors, for the quantized mixture-of-experts path only, the surface an mlx-rs user
+// programs against:
+//   Array                      a typed, shaped device buffer (mlx-rs/src/array/mod.rs:384-403)
+//   Exception / Result<T>      every operation returns a value or the library's message,
+//                              never throws on its own (mlx-rs/src/error.rs:226-280,
+//                              utils/guard.rs:20-49); Result::unwrap() throws for callers
+//                              who want exceptions
+//   ops::quantize / dequantize / gather_qmm
+//                              same argument order, optionals and defaults as
+//                              mlx-rs/src/ops/quantization.rs:50-83,124-158,160-230
+//   nn::SparseMoeBlock         forward(const Array&) -> Result<Array>, training_mode(bool):
+//                              the Module<&Array> contract, mlx-rs/src/module/module.rs:28-50
+// All arithmetic happens in libmi_moe.so; this file owns memory, shapes and error plumbing.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <numeric>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <utility>
+#include <variant>
+#include <vector>
+
+#include "mi_moe.h"
+
+namespace mi_moe {
+
+class Exception : public std::runtime_error {
+ public:
+  explicit Exception(const std::string &what) : std::runtime_error(what) {}
+  static Exception custom(const std::string &what) { return Exception(what); }
+};
+
+template <class T>
+class Result {
+ public:
+  Result(T v) : v_(std::move(v)) {}
+  Result(Exception e) : v_(std::move(e)) {}
+  bool is_ok() const { return v_.index() == 0; }
+  bool is_err() const { return !is_ok(); }
+  const Exception &error() const { return std::get<1>(v_); }
+  T &value() { return std::get<0>(v_); }
+  const T &value() const { return std::get<0>(v_); }
+  T unwrap() {
+    if (is_err()) throw error();
+    return std::move(std::get<0>(v_));
+  }
+
+ private:
+  std::variant<T, Exception> v_;
+};
+
+struct Unit {};
+
+namespace detail {
+inline Exception last_error(const char *who) {
+  return Exception(std::string(who) + ": " + mi_moe_last_error());
+}
+inline Exception hip_error(const char *who, hipError_t e) {
+  return Exception(std::string(who) + ": " + hipGetErrorString(e));
+}
+}  // namespace detail
+
+enum class Dtype { Bfloat16, Float32, Uint32 };
+inline size_t size_of(Dtype d) { return d == Dtype::Bfloat16 ? 2 : 4; }
+
+struct Stream {
+  hipStream_t handle = nullptr;  // nullptr = the default stream
+  void *as_ptr() const { return static_cast<void *>(handle); }
+};
+
+// A contiguous row-major device buffer with shape and dtype.  Copies share the allocation.
+class Array {
+ public:
+  Array() = default;
+  static Result<Array> empty(std::vector<int64_t> shape, Dtype dtype) {
+    Array a;
+    a.shape_ = std::move(shape);
+    a.dtype_ = dtype;
+    const size_t bytes = a.nbytes();
+    void *p = nullptr;
+    if (bytes) {
+      if (hipError_t e = hipMalloc(&p, bytes); e != hipSuccess)
+        return detail::hip_error("Array::empty", e);
+    }
+    a.mem_ = std::shared_ptr<void>(p, [](void *q) { if (q) (void)hipFree(q); });
+    return a;
+  }
+  // a view of memory somebody else owns (e.g. a tensor of the embedding framework)
+  static Array from_device_ptr(void *p, std::vector<int64_t> shape, Dtype dtype) {
+    Array a;
+    a.shape_ = std::move(shape);
+    a.dtype_ = dtype;
+    a.mem_ = std::shared_ptr<void>(p, [](void *) {});
+    return a;
+  }
+  static Result<Array> from_host(const void *src, std::vector<int64_t> shape, Dtype dtype,
+                                 Stream s = {}) {
+    auto r = empty(std::move(shape), dtype);
+    if (r.is_err()) return r;
+    if (size_t n = r.value().nbytes()) {
+      if (hipError_t e = hipMemcpyAsync(r.value().data(), src, n, hipMemcpyHostToDevice, s.handle);
+          e != hipSuccess)
+        return detail::hip_error("Array::from_host", e);
+      if (hipError_t e = hipStreamSynchronize(s.handle); e != hipSuccess)
+        return detail::hip_error("Array::from_host", e);
+    }
+    return r;
+  }
+  // eval + copy out, the counterpart of Array::as_slice
+  Result<Unit> to_host(void *dst, Stream s = {}) const {
+    if (hipError_t e = hipMemcpyAsync(dst, data(), nbytes(), hipMemcpyDeviceToHost, s.handle);
+        e != hipSuccess)
+      return detail::hip_error("Array::to_host", e);
+    if (hipError_t e = hipStreamSynchronize(s.handle); e != hipSuccess)
+      return detail::hip_error("Array::to_host", e);
+    return Unit{};
+  }
+  const std::vector<int64_t> &shape() const { return shape_; }
+  int64_t dim(int i) const { return shape_[i < 0 ? shape_.size() + i : i]; }
+  size_t ndim() const { return shape_.size(); }
+  Dtype dtype() const { return dtype_; }
+  int64_t size() const {
+    return std::accumulate(shape_.begin(), shape_.end(), (int64_t)1, std::multiplies<int64_t>());
+  }
+  size_t nbytes() const { return (size_t)size() * size_of(dtype_); }
+  void *data() const { return mem_.get(); }
+  template <class T> T *ptr() const { return static_cast<T *>(mem_.get()); }
+  Array reshape(std::vector<int64_t> shape) const {
+    Array a = *this;
+    a.shape_ = std::move(shape);
+    return a;
+  }
+
+ private:
+  std::vector<int64_t> shape_;
+  Dtype dtype_ = Dtype::Bfloat16;
+  std::shared_ptr<void> mem_;
+};
+
+namespace detail {
+inline std::optional<Exception> want(const Array &a, Dtype d, const char *who, const char *name) {
+  if (a.dtype() != d) return Exception(std::string(who) + ": " + name + " has the wrong dtype");
+  return std::nullopt;
+}
+}  // namespace detail
+
+namespace ops {
+
+constexpr int32_t DEFAULT_GROUP_SIZE = 64;  // mlx-rs/src/ops/quantization.rs:13-14
+constexpr int32_t DEFAULT_BITS = 4;
+
+// quantize(w, group_size, bits) -> (w_q, scales, biases); w: f32 [rows, cols]
+inline Result<std::tuple<Array, Array, Array>> quantize(const Array &w,
+                                                         std::optional<int32_t> group_size = {},
+                                                         std::optional<int32_t> bits = {},
+                                                         Stream s = {}) {
+  const int32_t g = group_size.value_or(DEFAULT_GROUP_SIZE), b = bits.value_or(DEFAULT_BITS);
+  if (auto e = detail::want(w, Dtype::Float32, "quantize", "w")) return *e;
+  if (w.ndim() != 2) return Exception("quantize: w must be a matrix");
+  const int64_t rows = w.dim(0), cols = w.dim(1);
+  // let the library judge the arguments before anything is allocated
+  if (g <= 0 || cols % g || (b != 2 && b != 4 && b != 8) || (g != 32 && g != 64 && g != 128)) {
+    if (mi_moe_quantize(nullptr, rows, cols, g, b, nullptr, nullptr, nullptr, nullptr))
+      return detail::last_error("quantize");
+  }
+  auto q = Array::empty({rows, cols * b / 32}, Dtype::Uint32);
+  auto sc = Array::empty({rows, cols / g}, Dtype::Bfloat16);
+  auto bi = Array::empty({rows, cols / g}, Dtype::Bfloat16);
+  if (q.is_err()) return q.error();
+  if (sc.is_err()) return sc.error();
+  if (bi.is_err()) return bi.error();
+  if (mi_moe_quantize(w.ptr<float>(), rows, cols, g, b, q.value().ptr<uint32_t>(),
+                      sc.value().ptr<uint16_t>(), bi.value().ptr<uint16_t>(), s.as_ptr()))
+    return detail::last_error("quantize");
+  return std::make_tuple(q.value(), sc.value(), bi.value());
+}
+
+// dequantize(w, scales, biases, group_size, bits) -> f32 [rows, cols]
+inline Result<Array> dequantize(const Array &w, const Array &scales, const Array &biases,
+                                std::optional<int32_t> group_size = {},
+                                std::optional<int32_t> bits = {}, Stream s = {}) {
+  const int32_t g = group_size.value_or(DEFAULT_GROUP_SIZE), b = bits.value_or(DEFAULT_BITS);
+  if (auto e = detail::want(w, Dtype::Uint32, "dequantize", "w")) return *e;
+  if (auto e = detail::want(scales, Dtype::Bfloat16, "dequantize", "scales")) return *e;
+  if (auto e = detail::want(biases, Dtype::Bfloat16, "dequantize", "biases")) return *e;
+  if (w.ndim() != 2 || (b != 2 && b != 4 && b != 8)) {
+    if (mi_moe_dequantize(nullptr, nullptr, nullptr, 1, 64, g, b, nullptr, nullptr))
+      return detail::last_error("dequantize");
+    return Exception("dequantize: w must be a matrix");
+  }
+  const int64_t rows = w.dim(0), cols = w.dim(1) * 32 / b;
+  auto out = Array::empty({rows, cols}, Dtype::Float32);
+  if (out.is_err()) return out;
+  if (mi_moe_dequantize(w.ptr<uint32_t>(), scales.ptr<uint16_t>(), biases.ptr<uint16_t>(), rows,
+                        cols, g, b, out.value().ptr<float>(), s.as_ptr()))
+    return detail::last_error("dequantize");
+  return out;
+}
+
+// gather_qmm(x, w, scales, biases, lhs_indices, rhs_indices, transpose, group_size, bits,
+// sorted_indices): x bf16 [x_batch, M, K]; w u32 [E, N, K*bits/32]; indices u32 [n_idx];
+// returns bf16 [n_idx, M, N].
+inline Result<Array> gather_qmm(const Array &x, const Array &w, const Array &scales,
+                                const Array *biases = nullptr, const Array *lhs_indices = nullptr,
+                                const Array *rhs_indices = nullptr,
+                                std::optional<bool> transpose = {},
+                                std::optional<int32_t> group_size = {},
+                                std::optional<int32_t> bits = {},
+                                std::optional<bool> sorted_indices = {}, Stream s = {}) {
+  const bool tr = transpose.value_or(true), sorted = sorted_indices.value_or(false);
+  const int32_t g = group_size.value_or(DEFAULT_GROUP_SIZE), b = bits.value_or(DEFAULT_BITS);
+  if (auto e = detail::want(x, Dtype::Bfloat16, "gather_qmm", "x")) return *e;
+  if (auto e = detail::want(w, Dtype::Uint32, "gather_qmm", "w")) return *e;
+  if (auto e = detail::want(scales, Dtype::Bfloat16, "gather_qmm", "scales")) return *e;
+  if (!biases) return Exception("gather_qmm: biases are required in affine mode");
+  if (!rhs_indices) return Exception("gather_qmm: rhs_indices is required");
+  if (x.ndim() != 3 || w.ndim() != 3)
+    return Exception("gather_qmm: x must be [batch, M, K] and w [E, N, K*bits/32]");
+  const int64_t n_idx = rhs_indices->size(), xb = x.dim(0);
+  const int32_t M = (int32_t)x.dim(1), K = (int32_t)x.dim(2);
+  const int32_t E = (int32_t)w.dim(0), N = (int32_t)w.dim(1);
+  size_t ws_bytes = 0;
+  if (mi_moe_gather_qmm_workspace_size(E, n_idx, M, &ws_bytes)) return detail::last_error("gather_qmm");
+  auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);
+  auto y = Array::empty({n_idx, (int64_t)M, (int64_t)N}, Dtype::Bfloat16);
+  if (ws.is_err()) return ws;
+  if (y.is_err()) return y;
+  if (mi_moe_gather_qmm(x.ptr<uint16_t>(), w.ptr<uint32_t>(), scales.ptr<uint16_t>(),
+                        biases->ptr<uint16_t>(), lhs_indices ? lhs_indices->ptr<uint32_t>() : nullptr,
+                        rhs_indices->ptr<uint32_t>(), n_idx, xb, M, N, K, E, tr ? 1 : 0, g, b,
+                        sorted ? 1 : 0, y.value().ptr<uint16_t>(), ws.value().data(),
+                        ws.value().nbytes(), s.as_ptr()))
+    return detail::last_error("gather_qmm");
+  // the workspace may be released only after the work that uses it has finished
+  if (hipError_t e = hipStreamSynchronize(s.handle); e != hipSuccess)
+    return detail::hip_error("gather_qmm", e);
+  return y;
+}
+
+}  // namespace ops
+
+namespace nn {
+
+// E quantized matrices with a leading expert axis: the fields of QuantizedLinear
+// (mlx-rs/src/nn/quantized.rs:254-279) per expert
+struct QuantizedSwitchLinear {
+  Array weight;  // u32 [E, N, K*bits/32]
+  Array scales;  // bf16 [E, N, K/group_size]
+  Array biases;  // bf16 [E, N, K/group_size]
+  mi_moe_qmat c_struct() const {
+    return {weight.ptr<uint32_t>(), scales.ptr<uint16_t>(), biases.ptr<uint16_t>()};
+  }
+};
+
+class SparseMoeBlock {
+ public:
+  SparseMoeBlock(const SparseMoeBlock &) = delete;
+  SparseMoeBlock &operator=(const SparseMoeBlock &) = delete;
+  SparseMoeBlock(SparseMoeBlock &&o) noexcept { *this = std::move(o); }
+  SparseMoeBlock &operator=(SparseMoeBlock &&o) noexcept {
+    if (this != &o) {
+      release();
+      cfg_ = o.cfg_;
+      gate_weight_ = std::move(o.gate_weight_);
+      router_bias_ = std::move(o.router_bias_);
+      gate_proj_ = std::move(o.gate_proj_);
+      up_proj_ = std::move(o.up_proj_);
+      down_proj_ = std::move(o.down_proj_);
+      workspace_ = std::move(o.workspace_);
+      workspace_tokens_ = o.workspace_tokens_;
+      handle_ = o.handle_;
+      training_ = o.training_;
+      o.handle_ = nullptr;
+    }
+    return *this;
+  }
+  ~SparseMoeBlock() { release(); }
+
+  // gate_weight: bf16 [E, H] (the router, a bias-free Linear); router_bias: f32 [E] or none
+  static Result<SparseMoeBlock> create(const mi_moe_config &cfg, Array gate_weight,
+                                       QuantizedSwitchLinear gate_proj,
+                                       QuantizedSwitchLinear up_proj,
+                                       QuantizedSwitchLinear down_proj,
+                                       std::optional<Array> router_bias = {}) {
+    SparseMoeBlock b;
+    b.cfg_ = cfg;
+    b.gate_weight_ = std::move(gate_weight);
+    b.router_bias_ = std::move(router_bias);
+    b.gate_proj_ = std::move(gate_proj);
+    b.up_proj_ = std::move(up_proj);
+    b.down_proj_ = std::move(down_proj);
+    mi_moe_weights w{b.gate_weight_.ptr<uint16_t>(),
+                     b.router_bias_ ? b.router_bias_->ptr<float>() : nullptr,
+                     b.gate_proj_.c_struct(), b.up_proj_.c_struct(), b.down_proj_.c_struct()};
+    if (mi_moe_create(&b.cfg_, &w, &b.handle_)) return detail::last_error("SparseMoeBlock");
+    return b;
+  }
+
+  // x: bf16 [..., H] -> bf16 [..., H]; asynchronous on the stream
+  Result<Array> forward(const Array &x, Stream s = {}, const mi_moe_debug_out *dbg = nullptr) {
+    if (auto e = detail::want(x, Dtype::Bfloat16, "forward", "x")) return *e;
+    if (x.ndim() < 1 || x.dim(-1) != cfg_.hidden)
+      return Exception("forward: last dimension must be " + std::to_string(cfg_.hidden));
+    const int64_t T = x.size() / cfg_.hidden;
+    if (auto r = reserve(T > 0 ? T : 1); r.is_err()) return r.error();
+    auto out = Array::empty(x.shape(), Dtype::Bfloat16);
+    if (out.is_err()) return out;
+    if (mi_moe_forward(handle_, x.ptr<uint16_t>(), T, out.value().ptr<uint16_t>(),
+                       workspace_.data(), workspace_.nbytes(), dbg, s.as_ptr()))
+      return detail::last_error("forward");
+    return out;
+  }
+
+  void training_mode(bool mode) { training_ = mode; }  // no layer here depends on it
+  const mi_moe_config &config() const { return cfg_; }
+
+  Result<size_t> workspace_bytes(int64_t tokens) const {
+    size_t n = 0;
+    if (mi_moe_workspace_size(&cfg_, tokens, &n)) return detail::last_error("workspace_size");
+    return n;
+  }
+  Result<Unit> reserve(int64_t tokens) {
+    if (tokens <= workspace_tokens_) return Unit{};
+    auto n = workspace_bytes(tokens);
+    if (n.is_err()) return n.error();
+    auto ws = Array::empty({(int64_t)(n.value() + 256 + 3) / 4}, Dtype::Uint32);
+    if (ws.is_err()) return ws.error();
+    workspace_ = ws.value();
+    workspace_tokens_ = tokens;
+    return Unit{};
+  }
+
+ private:
+  SparseMoeBlock() = default;
+  void release() {
+    if (handle_) mi_moe_destroy(handle_);
+    handle_ = nullptr;
+  }
+  mi_moe_config cfg_{};
+  Array gate_weight_;
+  std::optional<Array> router_bias_;
+  QuantizedSwitchLinear gate_proj_, up_proj_, down_proj_;
+  Array workspace_;
+  int64_t workspace_tokens_ = -1;
+  mi_moe_handle handle_ = nullptr;
+  bool training_ = false;
+};
+
+}  // namespace nn
+}  // namespace mi_moe

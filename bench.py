@@ -40,6 +40,7 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only-headline", action="store_true", help="run only the headline batch of the workload")
+    ap.add_argument("--batches", default="", help="comma-separated batch sizes to run besides the headline batch")
     ap.add_argument("--copy-probe", type=int, default=0,
                     help="first launch N plain 256 MiB copy kernels (a known-size reference for profiler counters)")
     return ap.parse_args()
@@ -84,6 +85,8 @@ def main():
     cfg_name, batches, headline, zipf_s, bound = WORKLOADS[args.workload]
     if args.only_headline:
         batches = [headline]
+    if args.batches:
+        batches = sorted(set(int(b) for b in args.batches.split(",")) | {headline})
     if args.copy_probe:
         # an elementwise kernel that reads 256 MiB and writes 256 MiB
         src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)

@@ -23,7 +23,11 @@
  *    where mlx-rs would call eval (mlx-rs/src/transforms/mod.rs:66-92);
  *  - the library keeps no input pointer after a call returns except the weight
  *    pointers registered with mi_moe_create; one handle is used by one host thread at
- *    a time (MLX itself is not thread safe, .github/workflows/validate.yml:46).
+ *    a time (MLX itself is not thread safe, .github/workflows/validate.yml:46), and
+ *    forwards through one handle must not overlap on the GPU (use one stream per handle):
+ *    a handle owns 260 bytes of device memory (arrival counters of the decode router
+ *    kernel), allocated by mi_moe_create on the current device and freed by
+ *    mi_moe_destroy.  No other entry point allocates device memory.
  *
  * Weight format = MLX "affine" quantisation (mlx-rs/src/ops/quantization.rs:31-47,
  * 85-87, 306-309): element c of a row lives in uint32 word c/(32/bits) at bit

@@ -121,6 +121,7 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
 struct mi_moe_s {
   mi_moe_config cfg;
   mi_moe_weights w;
+  uint32_t *counters = nullptr;  // device: arrival counters of the fused decode router, zero at rest
 };
 
 extern "C" {
@@ -149,11 +150,21 @@ int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_mo
   if (!h) return fail("create: out of host memory");
   h->cfg = *cfg;
   h->w = *weights;
+  // the only device memory the library owns: 260 bytes of counters per handle
+  const size_t cbytes = (size_t)(1 + kFusedRouterMaxTokens) * sizeof(uint32_t);
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&h->counters), cbytes);
+  if (e == hipSuccess) e = hipMemset(h->counters, 0, cbytes);
+  if (e != hipSuccess) {
+    if (h->counters) (void)hipFree(h->counters);
+    delete h;
+    return fail("create: device memory for the handle: %s", hipGetErrorString(e));
+  }
   *out = h;
   return 0;
 }
 
 int mi_moe_destroy(mi_moe_handle h) {
+  if (h && h->counters) (void)hipFree(h->counters);
   delete h;
   return 0;
 }
@@ -192,13 +203,24 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   } while (0)
   if (ev) MI_HIP(hipEventRecord(ev[0], st));
 
-  MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st));
-  MI_STAGE_DONE();
-  MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
-  MI_STAGE_DONE();
-  MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
-                         f.src_of, f.work, f.max_mtiles ? f.mtiles : nullptr, kBigThreshold, f.disp_scratch, st));
-  MI_STAGE_DONE();
+  if (router_fused_applies(T, c.n_experts, c.top_k)) {
+    // decode: one launch for the three stages (the stage times then all land in the first)
+    MI_HIP(launch_router_fused(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, c.top_k,
+                               c.score_mode, f.logits, f.topk_idx, f.topk_w, h->counters, f.counts, f.offsets,
+                               f.perm, f.inv_perm, f.src_of, f.work, f.max_mtiles ? f.mtiles : nullptr,
+                               kBigThreshold, st));
+    MI_STAGE_DONE();
+    MI_STAGE_DONE();
+    MI_STAGE_DONE();
+  } else {
+    MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st));
+    MI_STAGE_DONE();
+    MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
+    MI_STAGE_DONE();
+    MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
+                           f.src_of, f.work, f.max_mtiles ? f.mtiles : nullptr, kBigThreshold, f.disp_scratch, st));
+    MI_STAGE_DONE();
+  }
   const int max_active = (int)(P < c.n_experts ? P : c.n_experts);
   GroupedArgs a{};
   a.work = f.work;
@@ -277,7 +299,7 @@ int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t
       if (e != hipSuccess) rc = hip_fail("hipEventElapsedTime", e);
     }
   }
-  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) hipEventDestroy(ev[i]);
+  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) (void)hipEventDestroy(ev[i]);
   return rc;
 }
 

@@ -9,6 +9,7 @@ namespace mi_moe {
 constexpr int kWave = 64;
 constexpr int kBigThreshold = 48;  // segments with at least this many rows use the tiled kernel
 constexpr int kBigTileM = 256;     // rows per M tile of the tiled kernel
+constexpr int kFusedRouterMaxTokens = 64;  // up to here router + dispatch run as one launch
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
@@ -85,6 +86,19 @@ __device__ __forceinline__ float wave_max_f32(float v) {
   return v;
 }
 
+// ---------------------------------------------------------------- device-coherent accesses
+// A load that observes what other workgroups have written before an agent-scope release
+// (bypasses the per-CU cache).  Used for data produced earlier in the same launch.
+template <class T>
+__device__ __forceinline__ T load_agent(const T *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// The matching store: written through to where every workgroup's load_agent reads.
+template <class T>
+__device__ __forceinline__ void store_agent(T *p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ---------------------------------------------------------------- launchers (host)
 // Each returns hipSuccess or the launch error.  All pointers are device pointers.
 struct GroupedArgs {
@@ -117,6 +131,15 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
                            uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
                            uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
                            void *scratch, hipStream_t st);
+// decode-sized batches: logits + selection + dispatch in one launch.  counters: 1 +
+// kFusedRouterMaxTokens zero-initialised words that the kernel leaves zeroed again.
+bool router_fused_applies(int64_t T, int E, int k);
+hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const float *bias, int64_t T,
+                               int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx,
+                               uint16_t *topk_w, uint32_t *counters, uint32_t *counts,
+                               uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
+                               uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
+                               hipStream_t st);
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *out, hipStream_t st);

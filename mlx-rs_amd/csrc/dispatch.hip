@@ -7,194 +7,18 @@
 // computed from wave ballots in pair order, so the permutation is the one a stable
 // argsort gives, whatever order blocks and waves run in.  Also emits the list of
 // experts that received at least one pair (what the grouped products iterate over).
-#include "common.hpp"
+#include "dispatch_dev.hpp"
 
 namespace mi_moe {
 
-constexpr int kDispThreads = 1024;             // 16 waves
-constexpr int kDispWaves = kDispThreads / 64;  // pairs per chunk = 1024
-
-__device__ __forceinline__ uint64_t lanemask_lt() {
-  return (1ull << lane_id()) - 1ull;
-}
-
-// lanes (among `valid` ones) that hold the same expert id as this lane
-__device__ __forceinline__ uint64_t match_peers(uint32_t e, int nbits, bool valid) {
-  uint64_t peers = __ballot(valid);
-  for (int b = 0; b < nbits; ++b) {
-    const bool bit = (e >> b) & 1u;
-    const uint64_t bm = __ballot(valid && bit);
-    peers &= bit ? bm : ~bm;
-  }
-  return peers;
-}
-
-// exclusive scan of v[0..n) in LDS by one block of kDispThreads threads (n <= 1024);
-// tmp: n words.  Returns with v holding the exclusive scan and *total the sum.
-__device__ void block_exclusive_scan(uint32_t *v, uint32_t *tmp, int n, uint32_t *total) {
-  const int tid = threadIdx.x;
-  uint32_t mine = tid < n ? v[tid] : 0u;
-  uint32_t *src = v, *dst = tmp;
-  for (int off = 1; off < n; off <<= 1) {
-    uint32_t val = 0;
-    if (tid < n) val = src[tid] + (tid >= off ? src[tid - off] : 0u);
-    __syncthreads();
-    if (tid < n) dst[tid] = val;
-    __syncthreads();
-    uint32_t *t = src;
-    src = dst;
-    dst = t;
-  }
-  uint32_t incl = tid < n ? src[tid] : 0u;
-  __syncthreads();
-  if (tid < n) v[tid] = incl - mine;
-  if (tid == n - 1) *total = incl;
-  __syncthreads();
-}
-
-// Scatter the pairs [j0, j1) (j0 a multiple of 1024) given cur[e] = first free sorted
-// position of expert e for this range.  LDS: cur[E], wcnt[16*E].
-__device__ void scatter_range(const uint32_t *__restrict__ flat, int64_t j0, int64_t j1, int E,
-                              int nbits, int k_div, uint32_t *cur, uint32_t *wcnt,
-                              uint32_t *__restrict__ perm, uint32_t *__restrict__ inv_perm,
-                              uint32_t *__restrict__ src_of) {
-  const int tid = threadIdx.x, wave = tid >> 6;
-  for (int64_t c0 = j0; c0 < j1; c0 += kDispThreads) {
-    for (int i = tid; i < kDispWaves * E; i += kDispThreads) wcnt[i] = 0u;
-    __syncthreads();
-    const int64_t j = c0 + tid;
-    const bool valid = j < j1;
-    uint32_t e = valid ? flat[j] : 0u;
-    e = e < (uint32_t)E ? e : (uint32_t)E - 1u;  // out-of-range ids are clamped, never written past LDS
-    const uint64_t peers = match_peers(e, nbits, valid);
-    const uint32_t rank = __popcll(peers & lanemask_lt());
-    if (valid && rank == 0) wcnt[wave * E + e] = __popcll(peers);
-    __syncthreads();
-    for (int x = tid; x < E; x += kDispThreads) {
-      uint32_t run = cur[x];
-      for (int w = 0; w < kDispWaves; ++w) {
-        uint32_t c = wcnt[w * E + x];
-        wcnt[w * E + x] = run;
-        run += c;
-      }
-      cur[x] = run;
-    }
-    __syncthreads();
-    if (valid) {
-      const uint32_t pos = wcnt[wave * E + e] + rank;
-      perm[pos] = (uint32_t)j;
-      if (inv_perm) inv_perm[j] = pos;
-      if (src_of) src_of[pos] = (uint32_t)j / (uint32_t)k_div;
-    }
-    __syncthreads();
-  }
-}
-
-// Work records consumed by the grouped products: one 64-byte record per expert that received
-// rows, in ascending expert order, then records with count 0 up to n_experts.
-//   [0] expert id  [1] first sorted row  [2] row count  [3] 1 if [4..15] are filled
-//   [4..15] source row (pair index / k_div) of the first 12 rows of the segment
-constexpr int kWorkWords = 16;
-constexpr int kWorkSrc = 12;
-
-// Long segments (at least big_thr rows, big_thr > 0) go to the tiled MFMA kernel instead: they
-// are cut into M tiles of kBigTileM rows, listed in `mtiles`:
-//   mtiles[0] = number of tiles; tile i at mtiles[4 + 4 i] = {expert id, first sorted row, rows, 0}
-
-
-// counts -> offsets, work records and M tiles; runs in one block.  LDS cnt[E] in, cur[E] out.
-__device__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E,
-                              uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
-                              uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
-                              uint32_t big_thr, uint32_t *n_active_lds) {
-  __shared__ uint32_t total;
-  const int tid = threadIdx.x;
-  if (tid < E && counts) counts[tid] = cnt[tid];
-  __syncthreads();
-  block_exclusive_scan(cnt, tmp, E, &total);
-  if (tid < E) {
-    cur[tid] = cnt[tid];
-    if (offsets) offsets[tid] = cnt[tid];
-  }
-  if (tid == 0 && offsets) offsets[E] = total;
-  __syncthreads();
-  // experts with rows, in ascending order, by wave 0
-  if (tid < kWave) {
-    uint32_t base = 0, tbase = 0;
-    for (int e0 = 0; e0 < E; e0 += kWave) {
-      const int e = e0 + tid;
-      uint32_t c = 0;
-      if (e < E) c = (e + 1 < E ? cnt[e + 1] : total) - cnt[e];
-      const bool big = mtiles && big_thr != 0u && c >= big_thr;
-      const bool small = c != 0u && !big;
-      const uint64_t bm = __ballot(small);
-      if (small && work) {
-        uint32_t *rec = work + (size_t)(base + __popcll(bm & lanemask_lt())) * kWorkWords;
-        rec[0] = (uint32_t)e;
-        rec[1] = cnt[e];
-        rec[2] = c;
-        rec[3] = 0u;
-      }
-      base += __popcll(bm);
-      // M tiles of the long segments: exclusive scan of the tile counts over the wave
-      const uint32_t nt = big ? (c + kBigTileM - 1) / kBigTileM : 0u;
-      uint32_t incl = nt;
-      for (int d = 1; d < kWave; d <<= 1) {
-        const uint32_t v = __shfl_up(incl, d, kWave);
-        if (tid >= d) incl += v;
-      }
-      for (uint32_t i = 0; i < nt; ++i) {
-        uint32_t *rec = mtiles + 4 + (size_t)(tbase + incl - nt + i) * 4;
-        rec[0] = (uint32_t)e;
-        rec[1] = cnt[e] + i * kBigTileM;
-        rec[2] = c - i * kBigTileM < (uint32_t)kBigTileM ? c - i * kBigTileM : (uint32_t)kBigTileM;
-        rec[3] = 0u;
-      }
-      tbase += __shfl(incl, kWave - 1, kWave);
-    }
-    if (work)
-      for (int sl = base + tid; sl < E; sl += kWave) {
-        work[(size_t)sl * kWorkWords + 2] = 0u;
-        work[(size_t)sl * kWorkWords + 3] = 0u;
-      }
-    if (tid == 0) {
-      *n_active_lds = base;
-      if (mtiles) mtiles[0] = tbase;
-    }
-  }
-  __syncthreads();
-}
-
 // ---- one block does everything (decode-sized P)
 __global__ __launch_bounds__(kDispThreads) void dispatch_single_kernel(
-    const uint32_t *__restrict__ flat, int64_t P, int E, int nbits, int k_div,
+    const uint32_t *flat, int64_t P, int E, int nbits, int k_div,
     uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets, uint32_t *__restrict__ perm,
     uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of,
     uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles, uint32_t big_thr) {
   extern __shared__ uint32_t lds[];
-  __shared__ uint32_t n_active;
-  uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *wcnt = lds + 3 * E;
-  const int tid = threadIdx.x;
-  for (int i = tid; i < E; i += kDispThreads) cnt[i] = 0u;
-  __syncthreads();
-  for (int64_t j = tid; j < P; j += kDispThreads) {
-    const uint32_t e = flat[j];
-    atomicAdd(&cnt[e < (uint32_t)E ? e : (uint32_t)E - 1u], 1u);
-  }
-  __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, big_thr, &n_active);
-  scatter_range(flat, 0, P, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
-  // source rows of the first rows of every segment, so that a consumer needs one load
-  if (work) {
-    __threadfence_block();
-    __syncthreads();
-    for (int i = tid; i < (int)n_active * kWorkSrc; i += kDispThreads) {
-      uint32_t *rec = work + (size_t)(i / kWorkSrc) * kWorkWords;
-      const uint32_t j = i % kWorkSrc;
-      if (j < rec[2]) rec[4 + j] = perm[rec[1] + j] / (uint32_t)k_div;
-      if (j == 0) rec[3] = 1u;
-    }
-  }
+  dispatch_block(flat, P, E, nbits, k_div, lds, counts, offsets, perm, inv_perm, src_of, work, mtiles, big_thr);
 }
 
 // ---- three kernels for prefill-sized P: block b owns pairs [b*span, (b+1)*span)
@@ -241,7 +65,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
 }
 
 __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
-    const uint32_t *__restrict__ flat, int64_t P, int E, int nbits, int k_div, int64_t span,
+    const uint32_t *flat, int64_t P, int E, int nbits, int k_div, int64_t span,
     const uint32_t *__restrict__ blockbase, uint32_t *__restrict__ perm,
     uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of) {
   extern __shared__ uint32_t lds[];
@@ -254,7 +78,6 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
   scatter_range(flat, j0, j1, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
 }
 
-constexpr int64_t kSingleMaxP = 4096;
 constexpr int64_t kSpan = 2048;  // pairs per block in the multi-block path
 
 size_t dispatch_workspace_bytes(int E, int64_t P) {

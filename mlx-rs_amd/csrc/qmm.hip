@@ -425,9 +425,9 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // split K over the 4 waves of a block when there are too few row tiles to fill the chip
   const int64_t tiles = (int64_t)(a.N / 16) * a.max_active;
   const int chunks = a.K / (BITS == 4 ? 128 : 64);
-  int kw = 1;
-  if (tiles < 4096 && chunks >= 8) kw = 4;
-  else if (tiles < 8192 && chunks >= 4) kw = 2;
+  int kw = 1;  // measured on the 128-expert layer: 2 pays below ~2000 row tiles, 4 only when nearly empty
+  if (tiles < 256 && chunks >= 8) kw = 4;
+  else if (tiles < 2048 && chunks >= 4) kw = 2;
   const int nw = 4 / kw;
   dim3 grid((unsigned)((a.N + 16 * nw - 1) / (16 * nw)), (unsigned)a.max_active);
   if (kw == 4) qmm_small_kernel<BITS, GLU, 4><<<grid, 256, lds, st>>>(a, tt);

@@ -11,7 +11,7 @@
 //   logits  - fp64 accumulation of exact bf16*bf16 products, rounded fp64->fp32->bf16;
 //   softmax - det_expf terms, fp64 sum, one IEEE fp32 division, rounded to bf16;
 //   top-k   - total order (value descending, expert id ascending), slot 0 = best.
-#include "common.hpp"
+#include "router_dev.hpp"
 
 namespace mi_moe {
 
@@ -179,110 +179,14 @@ hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const flo
 }
 
 // ------------------------------------------------------------------ select
-// float -> unsigned key whose unsigned order is the float order; -0 is mapped to +0 so
-// that the two zeros tie (and the lower expert id wins) as they do in a float compare.
-__device__ __forceinline__ uint32_t ordered_key(float f) {
-  uint32_t u = __float_as_uint(f);
-  if (u == 0x80000000u) u = 0u;
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-__device__ __forceinline__ float key_to_float(uint32_t k) {
-  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
-  return __uint_as_float(u);
-}
-
-// One wave per token.  Lane l holds experts l, l+64, ... (NV of them).
+// One wave per token.
 template <int NV>
 __global__ __launch_bounds__(256) void router_select_kernel(
     const uint16_t *__restrict__ logits, int64_t T, int E, int k, int mode,
     uint32_t *__restrict__ topk_idx, uint16_t *__restrict__ topk_w) {
-  const int lane = lane_id();
   const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
-  const uint16_t *row = logits + t * E;
-
-  float g[NV], v[NV];
-  float m = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    int e = j * kWave + lane;
-    g[j] = e < E ? bf16_to_f32(row[e]) : -INFINITY;
-    m = fmaxf(m, g[j]);
-  }
-  if (mode != 2) {
-    m = wave_max_f32(m);
-    float ex[NV];
-    double sum = 0.0;
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      int e = j * kWave + lane;
-      ex[j] = e < E ? det_expf(g[j] - m) : 0.0f;
-      sum += (double)ex[j];
-    }
-    sum = wave_sum_f64(sum);
-    const float sf = (float)sum;
-#pragma unroll
-    for (int j = 0; j < NV; ++j) v[j] = bf16_to_f32(f32_to_bf16(ex[j] / sf));
-  } else {
-#pragma unroll
-    for (int j = 0; j < NV; ++j) v[j] = g[j];
-  }
-
-  // k rounds of wave-wide arg-max over 64-bit keys (value, then lower id)
-  uint32_t taken = 0;
-  uint32_t my_idx = 0;
-  float my_val = 0.0f;
-  for (int s = 0; s < k; ++s) {
-    uint32_t bk = 0, bi = 0;  // best key / inverted id of this lane
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      int e = j * kWave + lane;
-      if (e < E && !((taken >> j) & 1u)) {
-        uint32_t key = ordered_key(v[j]);
-        uint32_t inv = 0xffffffffu - (uint32_t)e;
-        if (key > bk || (key == bk && inv > bi)) {
-          bk = key;
-          bi = inv;
-        }
-      }
-    }
-#pragma unroll
-    for (int msk = 32; msk >= 1; msk >>= 1) {
-      uint32_t ok = __shfl_xor(bk, msk, kWave), oi = __shfl_xor(bi, msk, kWave);
-      if (ok > bk || (ok == bk && oi > bi)) {
-        bk = ok;
-        bi = oi;
-      }
-    }
-    const uint32_t win = 0xffffffffu - bi;
-    if ((int)(win & (kWave - 1)) == lane) taken |= 1u << (win >> 6);
-    if (lane == s) {
-      my_idx = win;
-      my_val = key_to_float(bk);
-    }
-  }
-
-  // scores; lane s holds slot s
-  float score;
-  if (mode == 2) {
-    const float mx = __shfl(my_val, 0, kWave);  // slot 0 is the largest logit
-    const float e_s = lane < k ? det_expf(my_val - mx) : 0.0f;
-    double sum = 0.0;
-    for (int s = 0; s < k; ++s) sum += (double)__shfl(e_s, s, kWave);
-    score = e_s / (float)sum;
-  } else {
-    score = my_val;
-    if (mode == 0) {
-      float sum = 0.0f;
-      for (int s = 0; s < k; ++s) sum += __shfl(my_val, s, kWave);
-      const float denom = bf16_to_f32(f32_to_bf16(sum));
-      score = my_val / denom;
-    }
-  }
-  if (lane < k) {
-    topk_idx[t * k + lane] = my_idx;
-    topk_w[t * k + lane] = f32_to_bf16(score);
-  }
+  select_wave<NV, false>(logits + t * E, E, k, mode, topk_idx + t * k, topk_w + t * k);
 }
 
 hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k, int mode,

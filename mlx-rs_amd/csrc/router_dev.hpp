@@ -1,0 +1,132 @@
+// Device-side building blocks of the router, shared by the stand-alone router kernels and the
+// fused decode router kernel: one logit per wave, and softmax / top-k / scores of one token per wave.
+#pragma once
+
+#include "common.hpp"
+
+namespace mi_moe {
+
+// logit of (token row xr, expert row wr): lanes split H in 16-byte pieces, exact bf16 x bf16
+// products accumulated in fp64, butterfly sum.  Every lane returns the sum.
+__device__ __forceinline__ double logit_wave(const uint16_t *__restrict__ xr,
+                                             const uint16_t *__restrict__ wr, int H) {
+  double acc = 0.0;
+  for (int h = lane_id() * 8; h < H; h += kWave * 8) {
+    const uint4 xv = *reinterpret_cast<const uint4 *>(xr + h);
+    const uint4 wv = *reinterpret_cast<const uint4 *>(wr + h);
+    const uint32_t xu[4] = {xv.x, xv.y, xv.z, xv.w}, wu[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      acc = __builtin_fma((double)bf16lo_to_f32(xu[q]), (double)bf16lo_to_f32(wu[q]), acc);
+      acc = __builtin_fma((double)bf16hi_to_f32(xu[q]), (double)bf16hi_to_f32(wu[q]), acc);
+    }
+  }
+  return wave_sum_f64(acc);
+}
+
+// float -> unsigned key whose unsigned order is the float order; -0 is mapped to +0 so
+// that the two zeros tie (and the lower expert id wins) as they do in a float compare.
+__device__ __forceinline__ uint32_t ordered_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_to_float(uint32_t k) {
+  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const uint32_t o = __shfl_xor(v, m, kWave);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+// Softmax, top-k and scores of one token by one wave.  Lane l holds experts l, l+64, ... (NV of
+// them).  COHERENT: the logits were written by other workgroups of the same launch.
+// The values the selection compares are exact in bf16 (rounded probabilities, or the logits
+// themselves), so value and expert id fit one 32-bit key: the upper half is the order-preserving
+// key of the bf16 value, the lower half 0xffff - expert id (lower id wins a tie).
+template <int NV, bool COHERENT>
+__device__ __forceinline__ void select_wave(const uint16_t *row, int E, int k, int mode,
+                                            uint32_t *idx_out,
+                                            uint16_t *__restrict__ w_out) {
+  const int lane = lane_id();
+  float g[NV], v[NV];
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int e = j * kWave + lane;
+    uint16_t bits = 0;
+    if (e < E) bits = COHERENT ? load_agent(row + e) : row[e];
+    g[j] = e < E ? bf16_to_f32(bits) : -INFINITY;
+    m = fmaxf(m, g[j]);
+  }
+  if (mode != 2) {
+    m = wave_max_f32(m);
+    float ex[NV];
+    double sum = 0.0;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = j * kWave + lane;
+      ex[j] = e < E ? det_expf(g[j] - m) : 0.0f;
+      sum += (double)ex[j];
+    }
+    sum = wave_sum_f64(sum);
+    const float sf = (float)sum;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[j] = bf16_to_f32(f32_to_bf16(ex[j] / sf));
+  } else {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[j] = g[j];
+  }
+
+  uint32_t key[NV];  // 0 = not a candidate (no real key is 0: the id half of a real key is >= 0xfe00)
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int e = j * kWave + lane;
+    key[j] = e < E ? ((ordered_key(v[j]) & 0xffff0000u) | (0xffffu - (uint32_t)e)) : 0u;
+  }
+  // k rounds of wave-wide arg-max
+  uint32_t my_key = 0;
+  for (int s = 0; s < k; ++s) {
+    uint32_t best = 0;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) best = key[j] > best ? key[j] : best;
+    best = wave_max_u32(best);
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (key[j] == best) key[j] = 0u;  // keys are distinct: exactly one lane drops its candidate
+    if (lane == s) my_key = best;
+  }
+  const uint32_t my_idx = 0xffffu - (my_key & 0xffffu);
+  const uint32_t hi = my_key & 0xffff0000u;
+  const float my_val = key_to_float((hi & 0x80000000u) ? hi : (hi | 0xffffu));
+
+  // scores; lane s holds slot s
+  float score;
+  if (mode == 2) {
+    const float mx = __shfl(my_val, 0, kWave);  // slot 0 is the largest logit
+    const float e_s = lane < k ? det_expf(my_val - mx) : 0.0f;
+    double sum = 0.0;
+    for (int s = 0; s < k; ++s) sum += (double)__shfl(e_s, s, kWave);
+    score = e_s / (float)sum;
+  } else {
+    score = my_val;
+    if (mode == 0) {
+      float sum = 0.0f;
+      for (int s = 0; s < k; ++s) sum += __shfl(my_val, s, kWave);
+      const float denom = bf16_to_f32(f32_to_bf16(sum));
+      score = my_val / denom;
+    }
+  }
+  if (lane < k) {
+    if (COHERENT) store_agent(idx_out + lane, my_idx);  // read by another workgroup of this launch
+    else idx_out[lane] = my_idx;
+    w_out[lane] = f32_to_bf16(score);
+  }
+}
+
+}  // namespace mi_moe

@@ -1,0 +1,99 @@
+// Decode-sized batches: router logits, selection and dispatch in ONE launch.
+//
+// The three stages are separated by grid-wide dependencies (a token's selection needs all of
+// its logits, the dispatch needs every token's selection).  Instead of ending the kernel at
+// each of them, the workgroup that arrives last does the next stage:
+//   - a workgroup computes 16 logits of one token (one per wave), publishes them, and counts
+//     itself in for that token; the one that completes the count selects for the token;
+//   - it then counts the token in; the workgroup that completes that count runs the dispatch.
+// Nobody waits: a workgroup that is not last simply exits, so the scheme cannot deadlock.
+// Data that crosses workgroups inside the launch (logits, selected experts, counters) is written
+// with device-coherent stores and read with device-coherent loads; a workgroup waits for its own
+// stores to be acknowledged before it counts itself in.  No cache-wide write-back or invalidate
+// is involved (on this chip those cost microseconds per workgroup).
+// The counters return to zero before the kernel ends, so the next launch finds them ready.
+// Results are those of the separate kernels bit for bit (same device functions, and none of
+// them depends on which workgroup runs it).
+#include "dispatch_dev.hpp"
+#include "router_dev.hpp"
+
+namespace mi_moe {
+
+// counters[0]: tokens selected; counters[1 + t]: logit workgroups of token t that have finished
+template <int NV>
+__global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
+    const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg, const float *__restrict__ bias,
+    int T, int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx, uint16_t *topk_w,
+    uint32_t *counters, int nbits, uint32_t *counts, uint32_t *offsets, uint32_t *perm,
+    uint32_t *inv_perm, uint32_t *src_of, uint32_t *work, uint32_t *mtiles, uint32_t big_thr) {
+  extern __shared__ uint32_t lds[];
+  __shared__ uint32_t last;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int t = blockIdx.x;
+  const int e = blockIdx.y * kDispWaves + wave;
+
+  if (e < E) {
+    double s = logit_wave(x + (int64_t)t * H, wg + (int64_t)e * H, H);
+    if (lane_id() == 0) {
+      if (bias) s += (double)bias[e];
+      store_agent(logits + (int64_t)t * E + e, f32_to_bf16((float)s));
+    }
+  }
+  // every wave's store has been acknowledged (workgroup-scope release = wait for own stores) ...
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0) {  // ... before the workgroup is counted in
+    const uint32_t old = __hip_atomic_fetch_add(counters + 1 + t, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = old == gridDim.y - 1;
+    if (last) store_agent(counters + 1 + t, 0u);
+  }
+  __syncthreads();
+  if (!last) return;
+
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  if (wave == 0)
+    select_wave<NV, true>(logits + (int64_t)t * E, E, k, mode, topk_idx + (int64_t)t * k,
+                          topk_w + (int64_t)t * k);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0) {
+    const uint32_t old = __hip_atomic_fetch_add(counters, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = old == gridDim.x - 1;
+    if (last) store_agent(counters, 0u);
+  }
+  __syncthreads();
+  if (!last) return;
+
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  dispatch_block(topk_idx, (int64_t)T * k, E, nbits, k, lds, counts, offsets, perm, inv_perm, src_of,
+                 work, mtiles, big_thr);
+}
+
+bool router_fused_applies(int64_t T, int E, int k) {
+  return T >= 1 && T <= kFusedRouterMaxTokens && T * k <= kSingleMaxP;
+}
+
+hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const float *bias, int64_t T,
+                               int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx,
+                               uint16_t *topk_w, uint32_t *counters, uint32_t *counts,
+                               uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
+                               uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
+                               hipStream_t st) {
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  dim3 grid((unsigned)T, (unsigned)((E + kDispWaves - 1) / kDispWaves));
+  const size_t lds = (size_t)(3 + kDispWaves) * E * sizeof(uint32_t);
+#define MI_FUSED(NV)                                                                              \
+  router_fused_kernel<NV><<<grid, kDispThreads, lds, st>>>(                                        \
+      x, wg, bias, (int)T, H, E, k, mode, logits, topk_idx, topk_w, counters, nbits, counts,      \
+      offsets, perm, inv_perm, src_of, work, mtiles, (uint32_t)big_thr)
+  if (E <= 64) MI_FUSED(1);
+  else if (E <= 128) MI_FUSED(2);
+  else if (E <= 256) MI_FUSED(4);
+  else MI_FUSED(8);
+#undef MI_FUSED
+  return hipGetLastError();
+}
+
+}  // namespace mi_moe

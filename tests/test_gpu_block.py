@@ -69,3 +69,27 @@ def test_run_to_run_identical(orc):
     blk = device_block(m, m.MoeConfig(256, 8, 2, 512), W)
     outs = [bits_u16(blk.forward(x)) for _ in range(3)]
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+def test_fused_router_equals_the_separate_kernels(orc):
+    """Up to 64 tokens the block runs logits + selection + dispatch as one launch; the stage-level
+    entry points run them as separate kernels.  Same integers and scores, call after call (the
+    launch leaves its arrival counters at zero), across batch sizes on both sides of the switch."""
+    import mlx_rs_amd as m
+    H, E, k, I = 256, 128, 8, 128
+    W = host_layer(orc, H, E, k, I, 4, 21, zipf_s=0.7)
+    blk = device_block(m, m.MoeConfig(H, E, k, I), W)
+    rw = bf16_tensor(W["router_w"], "cuda")
+    rb = torch.from_numpy(W["router_bias"]).cuda()
+    for rep, T in enumerate([1, 64, 3, 64, 17, 65, 2, 40, 1]):
+        print(f"fused router T={T}", flush=True)
+        x = bf16_tensor(host_tokens(orc, T, H, 100 + rep), "cuda")
+        _, dbg = blk.forward(x, debug=True)
+        inds, sc = m.ops.route(x, rw, k, 0, router_bias=rb)
+        counts, offsets, perm, inv = m.ops.dispatch(inds, E)
+        torch.cuda.synchronize()
+        for got, want, name in ((dbg["topk_idx"], inds, "topk_idx"), (dbg["counts"], counts, "counts"),
+                                (dbg["offsets"], offsets, "offsets"), (dbg["perm"], perm, "perm"),
+                                (dbg["inv_perm"], inv, "inv_perm")):
+            assert torch.equal(got.reshape(want.shape), want), f"{name} at T={T}"
+        assert torch.equal(dbg["topk_w"].view(torch.int16), sc.view(torch.int16)), f"scores at T={T}"

@@ -155,6 +155,18 @@ def main():
         eager_ms = time_steps(lambda i: blocks[i % n_layers].forward(x, out=outs[i % n_layers]),
                               args.steps, args.warmup, torch)
 
+        # spread of single steps (event pair around each eager step) and the cache-resident figure
+        # (one weight set only: at decode sizes it stays in the 256 MB Infinity Cache)
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for i, (e0, e1) in enumerate(evs):
+            e0.record()
+            blocks[i % n_layers].forward(x, out=outs[i % n_layers])
+            e1.record()
+        torch.cuda.synchronize()
+        per_step = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+        pct = lambda q: per_step[min(len(per_step) - 1, int(q * len(per_step)))]
+        resident_ms = time_steps(lambda i: blocks[0].forward(x, out=outs[0]), args.steps, args.warmup, torch)
+
         # per-kernel durations from HIP events on the launch stream, same K steps
         stage = [0.0] * m.capi.N_STAGES
         for i in range(args.steps):
@@ -172,6 +184,8 @@ def main():
         detail[str(T)] = {
             "tokens_per_s": T / (ms * 1e-3), "ms_per_step": ms, "ms_per_step_eager": eager_ms,
             "steps": steps_done, "active_experts": n_active,
+            "step_ms_p10_p50_p90_event_timed": [round(pct(0.1), 5), round(pct(0.5), 5), round(pct(0.9), 5)],
+            "ms_per_step_cache_resident_single_weight_set": resident_ms,
             "counts_max_mean_min": counts_stats[0],
             "layer_algorithmic_MB": alg_bytes / 1e6, "layer_GBps": alg_bytes / (ms * 1e-3) / 1e9,
             "layer_hbm_frac": alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
@@ -245,11 +259,24 @@ def cpu_baseline(cfg, block, T, seed, synth):
         oracle.moe_forward(ocfg, W, x, strict=True, n_threads=threads, debug=False)
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
+    t1 = []
+    for _ in range(2):  # the same layer on one thread
+        t0 = time.perf_counter()
+        oracle.moe_forward(ocfg, W, x, strict=True, n_threads=1, debug=False)
+        t1.append(time.perf_counter() - t0)
+    model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next(l.split(":", 1)[1].strip() for l in f if l.startswith("model name"))
+    except (OSError, StopIteration):
+        pass
     sample = "%d runs of the full layer at batch %d" % (len(times), Ts)
     if Ts != T:
         sample += " (token subsample of the %d-token workload; tokens/s is per token, so no scaling applied)" % T
     return {"value": Ts / med, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": sample + "; CPU oracle in op-by-op mode, OpenMP"}
+            "sample": sample + "; CPU oracle in op-by-op mode (restatement of the MLX CPU op sequence; MLX itself "
+                               "cannot be built offline), OpenMP",
+            "cpu_model": model, "single_thread_tokens_per_s": Ts / min(t1)}
 
 
 if __name__ == "__main__":

@@ -149,6 +149,17 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
                       int32_t group_size, int32_t bits, int32_t sorted_indices, uint16_t *y,
                       void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- dense quantized matmul (mlx_quantized_matmul, mlx-rs/src/ops/quantization.rs:91-122, as
+ * QuantizedLinear::forward calls it with transpose = true, mlx-rs/src/nn/quantized.rs:363-386):
+ * y (M x N) = x (M x K) . dequantize(w)^T on the same kernels as gather_qmm (one matrix, every row).
+ * x: bf16 [M, K]; w: [N, K*bits/32]; scales, biases: bf16 [N, K/group_size]; y: bf16 [M, N].
+ * transpose must be non-zero.  workspace >= mi_moe_quantized_matmul_workspace_size. */
+int mi_moe_quantized_matmul_workspace_size(int64_t M, int32_t K, int32_t bits, size_t *bytes);
+int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                            const uint16_t *biases, int64_t M, int32_t N, int32_t K,
+                            int32_t transpose, int32_t group_size, int32_t bits, uint16_t *y,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- R7 silu(gate) * up on bf16 arrays (mlx_sigmoid + mlx_multiply x2,
  * mlx-rs/src/nn/activation.rs:142-144,876-880).  The block itself fuses this into
  * the gate/up product; this entry point is the stand-alone op. ---- */

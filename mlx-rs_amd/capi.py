@@ -17,7 +17,8 @@ EXPORTS = (
     "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_forward_timed",
     "mi_moe_route_workspace_size",
     "mi_moe_route", "mi_moe_dispatch_workspace_size", "mi_moe_dispatch",
-    "mi_moe_gather_qmm_workspace_size", "mi_moe_gather_qmm", "mi_moe_swiglu", "mi_moe_combine",
+    "mi_moe_gather_qmm_workspace_size", "mi_moe_gather_qmm",
+    "mi_moe_quantized_matmul_workspace_size", "mi_moe_quantized_matmul", "mi_moe_swiglu", "mi_moe_combine",
     "mi_moe_quantize", "mi_moe_dequantize",
 )
 
@@ -90,6 +91,8 @@ def load_library():
         "mi_moe_gather_qmm_workspace_size": [i32, i64, i32, C.POINTER(sz)],
         "mi_moe_gather_qmm": [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, i32, i32, i32,
                               i32, vp, vp, sz, vp],
+        "mi_moe_quantized_matmul_workspace_size": [i64, i32, i32, C.POINTER(sz)],
+        "mi_moe_quantized_matmul": [vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, vp, sz, vp],
         "mi_moe_swiglu": [vp, vp, i64, vp, vp],
         "mi_moe_combine": [vp, vp, vp, i64, i32, i32, vp, vp],
         "mi_moe_quantize": [vp, i64, i64, i32, i32, vp, vp, vp, vp],

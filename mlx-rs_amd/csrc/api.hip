@@ -426,6 +426,66 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   return 0;
 }
 
+static size_t qmm_dense_bytes(int64_t M, int32_t K, int32_t bits, size_t *mt_words) {
+  const size_t ntiles = (size_t)((M + kBigTileM - 1) / kBigTileM);
+  *mt_words = 4 + 4 * ntiles;
+  size_t b = 256 + 64 + *mt_words * 4 + 256;
+  if (bits == 4 && M >= kBigThreshold) b += (size_t)M * K * 2 + 256;
+  return b;
+}
+
+int mi_moe_quantized_matmul_workspace_size(int64_t M, int32_t K, int32_t bits, size_t *bytes) {
+  if (!bytes) return fail("quantized_matmul_workspace_size: bytes is NULL");
+  if (M < 0 || K <= 0 || M * (int64_t)K > (int64_t)1 << 40) return fail("quantized_matmul_workspace_size: bad sizes");
+  size_t mt = 0;
+  *bytes = qmm_dense_bytes(M, K, bits, &mt);
+  return 0;
+}
+
+int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                            const uint16_t *biases, int64_t M, int32_t N, int32_t K, int32_t transpose,
+                            int32_t group_size, int32_t bits, uint16_t *y, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+  if (!transpose) return fail("quantized_matmul: transpose = false is not supported (weights must be [N, K*bits/32])");
+  if (bits != 4 && bits != 8) return fail("quantized_matmul: bits must be 4 or 8, got %d", bits);
+  if (group_size != 64) return fail("quantized_matmul: group_size must be 64, got %d", group_size);
+  if (K <= 0 || K % 64) return fail("quantized_matmul: K must be a positive multiple of 64, got %d", K);
+  if (bits == 4 && K % 128) return fail("quantized_matmul: 4-bit weights need K to be a multiple of 128, got %d", K);
+  if (N <= 0 || N % 16) return fail("quantized_matmul: N must be a positive multiple of 16, got %d", N);
+  if (M < 0 || M > (int64_t)1 << 30) return fail("quantized_matmul: row count out of range");
+  if (M == 0) return 0;
+  if (!x || !w || !scales || !biases || !y) return fail("quantized_matmul: x, w, scales, biases and y must be non-NULL");
+  if (!aligned16(x) || !aligned16(w) || !aligned16(scales) || !aligned16(biases) || !aligned16(y))
+    return fail("quantized_matmul: pointers must be 16-byte aligned");
+  size_t mt_words = 0;
+  const size_t need = qmm_dense_bytes(M, K, bits, &mt_words);
+  if (!workspace || workspace_bytes < need) return fail("quantized_matmul: workspace too small (need %zu bytes)", need);
+  Carver cv(workspace);
+  uint32_t *work = cv.take<uint32_t>(16);
+  uint32_t *mtiles = cv.take<uint32_t>(mt_words);
+  const bool big = M >= kBigThreshold;
+  uint16_t *xperm = (bits == 4 && big) ? cv.take<uint16_t>((size_t)M * K) : nullptr;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MI_HIP(launch_dense_records(M, kBigThreshold, work, mtiles, st));
+  if (xperm) MI_HIP(launch_pair_rows(x, M, K, xperm, st));
+  GroupedArgs a{};
+  a.x = x;
+  a.x_perm = bits == 4 ? xperm : x;
+  a.work = work;
+  a.max_active = 1;
+  a.mtiles = big ? mtiles : nullptr;
+  a.max_mtiles = big ? (int)((M + kBigTileM - 1) / kBigTileM) : 0;
+  a.w0 = w; a.s0 = scales; a.b0 = biases;
+  a.y = y;
+  a.N = N;
+  a.K = K;
+  a.bits = bits;
+  a.total_rows = M;
+  a.max_rows_per_expert = M;
+  MI_HIP(launch_grouped_qmm(a, false, st));
+  return 0;
+}
+
 int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out, void *stream) {
   if (n < 0) return fail("swiglu: negative element count");
   if (n == 0) return 0;

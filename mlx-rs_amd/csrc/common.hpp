@@ -146,6 +146,7 @@ hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *ou
 hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
                            uint32_t *work, hipStream_t st);
+hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t *mtiles, hipStream_t st);
 hipError_t launch_swiglu(const uint16_t *g, const uint16_t *u, int64_t n, uint16_t *out,
                          hipStream_t st);
 hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,

@@ -109,6 +109,29 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
   return hipGetLastError();
 }
 
+// One dense segment (a plain quantized matmul: every row goes to matrix 0): the work record or, from
+// big_thr rows on, the M tiles of the tiled kernel.
+__global__ void dense_records_kernel(uint32_t M, uint32_t big_thr, uint32_t *__restrict__ work,
+                                     uint32_t *__restrict__ mtiles) {
+  const uint32_t tid = threadIdx.x;
+  const bool big = big_thr != 0u && M >= big_thr;
+  const uint32_t ntiles = big ? (M + kBigTileM - 1) / kBigTileM : 0u;
+  if (tid < kWorkWords) work[tid] = (tid == 2 && !big) ? M : 0u;  // {expert 0, row 0, M rows, no inline rows}
+  if (tid == 0) mtiles[0] = ntiles;
+  for (uint32_t i = tid; i < ntiles; i += blockDim.x) {
+    uint32_t *rec = mtiles + 4 + (size_t)i * 4;
+    rec[0] = 0u;
+    rec[1] = i * kBigTileM;
+    rec[2] = M - i * kBigTileM < (uint32_t)kBigTileM ? M - i * kBigTileM : (uint32_t)kBigTileM;
+    rec[3] = 0u;
+  }
+}
+
+hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t *mtiles, hipStream_t st) {
+  dense_records_kernel<<<1, 256, 0, st>>>((uint32_t)M, (uint32_t)big_thr, work, mtiles);
+  return hipGetLastError();
+}
+
 // Row maps for the stand-alone gather_qmm: sorted position q of index j = perm[q]
 // covers M rows; x rows come from lhs[j]*M + m, outputs go to j*M + m.
 __global__ void row_maps_kernel(const uint32_t *__restrict__ perm, const uint32_t *__restrict__ lhs,

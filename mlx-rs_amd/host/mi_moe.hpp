@@ -206,6 +206,37 @@ inline Result<Array> dequantize(const Array &w, const Array &scales, const Array
   return out;
 }
 
+// quantized_matmul(x, w, scales, biases, transpose, group_size, bits): x bf16 [M, K]; w u32
+// [N, K*bits/32]; returns bf16 [M, N].  The reference's default is transpose = false; only the
+// transposed layout (the one QuantizedLinear uses) is implemented, so it is the default here.
+inline Result<Array> quantized_matmul(const Array &x, const Array &w, const Array &scales,
+                                      const Array *biases = nullptr, std::optional<bool> transpose = {},
+                                      std::optional<int32_t> group_size = {},
+                                      std::optional<int32_t> bits = {}, Stream s = {}) {
+  const bool tr = transpose.value_or(true);
+  const int32_t g = group_size.value_or(DEFAULT_GROUP_SIZE), b = bits.value_or(DEFAULT_BITS);
+  if (auto e = detail::want(x, Dtype::Bfloat16, "quantized_matmul", "x")) return *e;
+  if (auto e = detail::want(w, Dtype::Uint32, "quantized_matmul", "w")) return *e;
+  if (auto e = detail::want(scales, Dtype::Bfloat16, "quantized_matmul", "scales")) return *e;
+  if (!biases) return Exception("quantized_matmul: biases are required in affine mode");
+  if (x.ndim() != 2 || w.ndim() != 2) return Exception("quantized_matmul: x must be [M, K] and w [N, K*bits/32]");
+  const int64_t M = x.dim(0);
+  const int32_t K = (int32_t)x.dim(1), N = (int32_t)w.dim(0);
+  size_t ws_bytes = 0;
+  if (mi_moe_quantized_matmul_workspace_size(M, K, b, &ws_bytes)) return detail::last_error("quantized_matmul");
+  auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);
+  auto y = Array::empty({M, (int64_t)N}, Dtype::Bfloat16);
+  if (ws.is_err()) return ws;
+  if (y.is_err()) return y;
+  if (mi_moe_quantized_matmul(x.ptr<uint16_t>(), w.ptr<uint32_t>(), scales.ptr<uint16_t>(),
+                              biases->ptr<uint16_t>(), M, N, K, tr ? 1 : 0, g, b, y.value().ptr<uint16_t>(),
+                              ws.value().data(), ws.value().nbytes(), s.as_ptr()))
+    return detail::last_error("quantized_matmul");
+  if (hipError_t e = hipStreamSynchronize(s.handle); e != hipSuccess)
+    return detail::hip_error("quantized_matmul", e);
+  return y;
+}
+
 // gather_qmm(x, w, scales, biases, lhs_indices, rhs_indices, transpose, group_size, bits,
 // sorted_indices): x bf16 [x_batch, M, K]; w u32 [E, N, K*bits/32]; indices u32 [n_idx];
 // returns bf16 [n_idx, M, N].

@@ -90,6 +90,30 @@ def gather_qmm(x, w, scales, biases, lhs_indices=None, rhs_indices=None, transpo
     return y
 
 
+def quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4):
+    """ops::quantized_matmul (mlx-rs/src/ops/quantization.rs:91-122) the way QuantizedLinear calls
+    it (transpose = true, mlx-rs/src/nn/quantized.rs:363-386; the op's own default is false, which
+    this build does not implement).  x: bf16 [..., K]; w: int32 [N, K*bits/32]; returns bf16 [..., N]."""
+    lib = load_library()
+    _need(x, torch.bfloat16, "x")
+    _need(w, torch.int32, "w")
+    if w.dim() != 2 or x.dim() < 1:
+        raise capi.MoeError("quantized_matmul: x must be [..., K] and w [N, K*bits/32]")
+    K = x.shape[-1]
+    N = w.shape[0]
+    x2 = x.reshape(-1, K)
+    M = x2.shape[0]
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    need = C.c_size_t()
+    check(lib.mi_moe_quantized_matmul_workspace_size(M, K, bits, C.byref(need)))
+    ws = _workspace(need.value, x.device)
+    check(lib.mi_moe_quantized_matmul(_ptr(x2), _ptr(w), _ptr(_need(scales, torch.bfloat16, "scales")),
+                                      _ptr(_need(biases, torch.bfloat16, "biases")), M, N, K,
+                                      1 if transpose else 0, group_size, bits, _ptr(y), _ptr(ws), ws.numel(),
+                                      _stream()))
+    return y.reshape(*x.shape[:-1], N)
+
+
 def route(x, router_w, top_k, score_mode=capi.SCORE_SOFTMAX_THEN_TOPK_RENORM, router_bias=None,
           return_logits=False):
     """Gate Linear + softmax(precise) + top-k + scores in one call (what an mlx-lm MoE block

@@ -156,3 +156,34 @@ def test_errors_reach_the_caller(m):
     with pytest.raises(m.MoeError, match="top_k"):
         m.ops.route(torch.zeros((4, 128), dtype=torch.bfloat16, device="cuda"),
                     torch.zeros((8, 128), dtype=torch.bfloat16, device="cuda"), 9)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M", [1, 5, 47, 48, 300])
+def test_quantized_matmul_equals_matmul_on_dequantized(orc, bits, M):
+    """The identity of the reference's test_quantized_matmul (mlx-rs/src/ops/quantization.rs:318-342),
+    in the transposed layout QuantizedLinear uses: qmm(x, w_q, s, b) == x @ dequantize(w_q, s, b)^T.
+    Rows below 48 run on the streaming kernel, from 48 on on the tiled one."""
+    import mlx_rs_amd as m
+    rng = np.random.default_rng(50 + M)
+    N, K = 192, 256
+    w = (rng.normal(0, 1, (N, K)) / np.sqrt(K)).astype(np.float32)
+    q, s, b = orc.quantize(w, bits, 64)
+    x = orc.f32_to_bf16((rng.normal(0, 1, (M, K))).astype(np.float32))
+    print(f"quantized_matmul bits={bits} M={M}", flush=True)
+    y = m.ops.quantized_matmul(bf16_tensor(x, "cuda"), i32_tensor(q, "cuda"), bf16_tensor(s, "cuda"),
+                               bf16_tensor(b, "cuda"), True, 64, bits)
+    torch.cuda.synchronize()
+    w_hat = orc.dequantize(q, s, b, bits, 64).astype(np.float64)
+    ref = f32_of_bits(x).astype(np.float64) @ w_hat.T
+    got = f32_of_bits(bits_u16(y)).astype(np.float64)
+    assert got.shape == ref.shape
+    assert np.abs(got - ref).max() <= 2e-2
+    assert np.linalg.norm(got - ref) / np.linalg.norm(ref) <= 1e-2
+    # and the oracle's gather_qmm with a single matrix agrees with the same identity
+    yo = orc.gather_qmm(x.reshape(M, 1, K), q[None], s[None], b[None], None, np.zeros(M, np.uint32),
+                        bits=bits, want="f32").reshape(M, N)
+    assert np.abs(yo - ref).max() <= 1e-4
+    with pytest.raises(m.MoeError, match="transpose"):
+        m.ops.quantized_matmul(bf16_tensor(x, "cuda"), i32_tensor(q, "cuda"), bf16_tensor(s, "cuda"),
+                               bf16_tensor(b, "cuda"), False, 64, bits)

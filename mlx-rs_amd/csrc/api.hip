@@ -103,7 +103,10 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.work = cv.take<uint32_t>((size_t)c.n_experts * 16);
   // M tiles of the tiled kernel: at most one partial tile per long segment plus P / tile full ones
   // (a segment is at most T rows long: no token picks an expert twice)
-  f.max_mtiles = T >= kBigThreshold ? (int)(P / kBigTileM + (P / kBigThreshold < c.n_experts ? P / kBigThreshold : c.n_experts)) : 0;
+  // (the tiled kernel reads scales in 8-byte pieces: rows of scales must be 4-byte aligned, i.e.
+  // an even number of groups per row; other shapes stay on the streaming kernel)
+  const bool tiled_ok = (c.hidden / 64) % 2 == 0 && (c.intermediate / 64) % 2 == 0;
+  f.max_mtiles = T >= kBigThreshold && tiled_ok ? (int)(P / kBigTileM + (P / kBigThreshold < c.n_experts ? P / kBigThreshold : c.n_experts)) : 0;
   f.mtiles = cv.take<uint32_t>(4 + (size_t)f.max_mtiles * 4);
   f.perm = cv.take<uint32_t>((size_t)P);
   f.inv_perm = cv.take<uint32_t>((size_t)P);
@@ -463,10 +466,10 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
   Carver cv(workspace);
   uint32_t *work = cv.take<uint32_t>(16);
   uint32_t *mtiles = cv.take<uint32_t>(mt_words);
-  const bool big = M >= kBigThreshold;
+  const bool big = M >= kBigThreshold && (K / 64) % 2 == 0;
   uint16_t *xperm = (bits == 4 && big) ? cv.take<uint16_t>((size_t)M * K) : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  MI_HIP(launch_dense_records(M, kBigThreshold, work, mtiles, st));
+  MI_HIP(launch_dense_records(M, big ? kBigThreshold : 0, work, mtiles, st));
   if (xperm) MI_HIP(launch_pair_rows(x, M, K, xperm, st));
   GroupedArgs a{};
   a.x = x;

@@ -3,18 +3,25 @@
 // Same contract as the small-segment kernel (mlx_gather_qmm with transpose = true,
 // mlx-rs/src/ops/quantization.rs:160-230; with GLU also nn::silu and multiply,
 // nn/activation.rs:142-144,876-880), restricted to the segments the dispatch cut into M tiles
-// of 256 rows.  A block computes a 256-token x 128-weight-row tile:
-//   * weights stream from HBM as packed codes (one 16-byte load per thread and 64-wide K step),
+// of 256 rows.  A block of 8 waves computes a 256-token x 256-weight-row tile:
+//   * weights stream from HBM as packed codes (one 8- or 16-byte load per thread and K step; scales
+//     and biases in 8-byte pieces that last 16 K steps),
 //     are dequantised ONCE per block to bf16 (w_hat = s q + b, fp32 fma, one rounding) and
 //     parked in LDS, so the cost of unpacking is shared by the 256 token rows of the tile;
 //   * the token rows are gathered through the sorted-row -> source-row map straight into LDS
 //     (no materialised gather);
-//   * 4 waves (2 x 2) run v_mfma_f32_32x32x16_bf16 on 128 x 64 sub-tiles, fp32 accumulators;
-//   * with GLU the 128 weight rows are 64 gate rows and the matching 64 up rows, each wave owns
+//   * 8 waves (2 x 4) run v_mfma_f32_32x32x16_bf16 on 128 x 64 sub-tiles, fp32 accumulators;
+//   * with GLU the 256 weight rows are 128 gate rows and the matching 128 up rows, each wave owns
 //     32 + 32 of them, and the epilogue writes silu(gate) * up without either product ever
 //     reaching memory.
-// The next K step's global loads are in flight while the current one is multiplied.
+// Three K steps of global loads are in flight while the current one is multiplied.
+#include <type_traits>
+
 #include "common.hpp"
+
+#ifndef MI_MOE_WEAVE
+#define MI_MOE_WEAVE 1
+#endif
 
 namespace mi_moe {
 
@@ -22,7 +29,9 @@ namespace {
 
 constexpr int BM = kBigTileM;  // token rows per block
 constexpr int BK = 32;         // K step (two steps per quantisation group)
-constexpr int BR = 128;        // weight rows per block (GLU: 64 gate + 64 up)
+constexpr int BR = 256;        // weight rows per block (GLU: 128 gate + 128 up)
+constexpr int NTHREADS = 512;  // 8 waves: 2 (token halves) x 4 (weight-row quarters)
+constexpr int DEPTH = 4;       // register stages: three K steps of global loads in flight
 
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
@@ -38,15 +47,23 @@ __device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
 
 // LDS tiles hold rows of 32 bf16 (four 16-byte chunks) at a stride of 80 bytes: consecutive
 // rows reading the same chunk start 20 banks apart, which keeps 16-byte reads of 8 or 16
-// consecutive rows free of bank conflicts (measured: SQ_LDS_BANK_CONFLICT = 0).
+// consecutive rows clear of each other.
 constexpr int LDR = 5;  // row stride in uint4 units
 __device__ __forceinline__ int tile_off(int row, int chunk) { return row * LDR + chunk; }
+constexpr size_t kLargeLdsBytes = (size_t)2 * (BM + BR) * LDR * 16;  // two steps of A and B tiles
 
 }  // namespace
 
+// Why this shape.  Measured on the 256 x 128 / 4-wave predecessor of this kernel: its global loads
+// alone (no LDS, no MFMA) took 0.9 us per K step against 0.43 us of MFMA work, because a step could
+// not start before loads issued only one to two steps earlier had come back (~1 us under load).
+// A 256 x 256 tile halves the activation bytes per MFMA, 512 threads halve the staging registers a
+// thread needs per step, and the registers saved pay for four stages, i.e. three steps of loads in
+// flight.  Per-step 2-byte gathers of scales and biases (more expensive than all other loads of
+// that kernel together) became one 8-byte load per 16 steps.
 template <int BITS, bool GLU>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qmm_large_kernel(GroupedArgs a, int n_ntiles) {
-  constexpr int NI = GLU ? 64 : 128;  // distinct output columns per block
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void qmm_large_kernel(GroupedArgs a, int n_ntiles) {
+  constexpr int NI = GLU ? 128 : 256;  // distinct output columns per block
 
   // block -> (M tile, N tile): blocks of one M tile share the gathered token rows, so they
   // are given consecutive ids on ONE XCD (ids are dealt round-robin over the 8 XCDs)
@@ -62,18 +79,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave >> 2, wn = wave & 3;
   const int N = a.N, K = a.K;
   const int n0 = nt * NI;
   const int row_bytes = K * BITS / 8, gpr = K / 64;
 
-  __shared__ u32x4_t As[2][BM * LDR];
-  __shared__ u32x4_t Bs[2][BR * LDR];
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  u32x4_t *const lds = reinterpret_cast<u32x4_t *>(lds_raw);
+  // [A step-parity 0][A parity 1][B parity 0][B parity 1]
+  auto As = [&](int buf) { return lds + buf * (BM * LDR); };
+  auto Bs = [&](int buf) { return lds + 2 * BM * LDR + buf * (BR * LDR); };
 
   // ---- global -> register stage
   // A: the activations arrive with every 8-block already in the (x0,x4,x1,x5,x2,x6,x3,x7) order
   // of the nibble unpacking (4-bit), so a row chunk is copied as it is.  Thread: chunk acp of
-  // rows arg + 64 j.
+  // rows arg and arg + 128.
   const int acp = tid & 3, arg = tid >> 2;
   auto a_row_ptr = [&](int tr) {
     tr = tr < rows ? tr : rows - 1;  // rows past the segment repeat its last row (never stored)
@@ -81,76 +101,88 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int64_t src = a.src_rows ? (int64_t)a.src_rows[r] : r;
     return a.x_perm + src * K + acp * 8;
   };
-  const uint16_t *const arow[4] = {a_row_ptr(arg), a_row_ptr(arg + 64), a_row_ptr(arg + 128), a_row_ptr(arg + 192)};
-  // B: thread covers 16 codes (half a K step) of weight row br; waves 0,1 / 2,3 hold gate / up
+  const uint16_t *const arow[2] = {a_row_ptr(arg), a_row_ptr(arg + 128)};
+  // B: thread covers 16 codes (half a K step) of weight row br; waves 0-3 / 4-7 hold gate / up
   const int br = tid >> 1, bh = tid & 1;
-  const int mat = GLU ? (wave >> 1) : 0;  // wave-uniform
-  const int nrow = GLU ? n0 + (br & 63) : n0 + br;  // rows >= N read zeros through the descriptor
+  const int mat = GLU ? (wave >> 2) : 0;  // wave-uniform
+  const int nrow = GLU ? n0 + (br & 127) : n0 + br;  // rows >= N read zeros through the descriptor
   const int64_t ebase = (int64_t)e * N;
   const __amdgpu_buffer_rsrc_t wr = make_rsrc((mat ? a.w1 : a.w0) + ebase * (row_bytes / 4), (uint32_t)N * row_bytes);
   const __amdgpu_buffer_rsrc_t sr = make_rsrc((mat ? a.s1 : a.s0) + ebase * gpr, (uint32_t)N * gpr * 2);
   const __amdgpu_buffer_rsrc_t brs = make_rsrc((mat ? a.b1 : a.b0) + ebase * gpr, (uint32_t)N * gpr * 2);
   const uint32_t w_voff = (uint32_t)nrow * row_bytes + bh * (BITS == 4 ? 8 : 16);
-  const uint32_t g_voff = (uint32_t)nrow * gpr * 2;
-
-  // Two sets of staging registers (plain scalars: they must not end up in scratch or LDS), so
-  // that global loads are issued two K steps before their data is needed.
-  struct Stage {
-    u32x4_t a0, a1, a2, a3;
-    uint32_t b0w, b1w, b2w, b3w;  // 4-bit: two words used
-    uint32_t sreg, bireg;
+  // scales / biases: a thread keeps a window of 8 groups (16 K steps) of its row, half of it in
+  // its own registers (groups 4 bh .. 4 bh + 3 of the window, one 8-byte load per tensor) and half
+  // in its neighbour's (the other thread of the row).
+  const uint32_t g_voff = (uint32_t)nrow * gpr * 2 + bh * 8;
+  struct SbWindow {
+    u32x2_t s, b;
   };
+  auto load_window = [&](int w) __attribute__((always_inline)) {
+    SbWindow v;
+    v.s = __builtin_amdgcn_raw_buffer_load_b64(sr, g_voff, w * 16, 0);
+    v.b = __builtin_amdgcn_raw_buffer_load_b64(brs, g_voff, w * 16, 0);
+    return v;
+  };
+
+  struct Stage {
+    u32x4_t a0, a1;
+    u32x4_t bw;  // 4-bit: two words used
+  };
+  // every load is unconditional (indices are clamped by the caller): the compiler can then count
+  // the loads in flight and wait for exactly the stage it needs
   auto gload = [&](int ks, Stage &R) __attribute__((always_inline)) {
     R.a0 = *reinterpret_cast<const u32x4_t *>(arow[0] + ks * BK);
     R.a1 = *reinterpret_cast<const u32x4_t *>(arow[1] + ks * BK);
-    R.a2 = *reinterpret_cast<const u32x4_t *>(arow[2] + ks * BK);
-    R.a3 = *reinterpret_cast<const u32x4_t *>(arow[3] + ks * BK);
     if constexpr (BITS == 4) {
       const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(wr, w_voff, ks * 16, 0);
-      R.b0w = v[0];
-      R.b1w = v[1];
+      R.bw[0] = v[0];
+      R.bw[1] = v[1];
     } else {
-      const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(wr, w_voff, ks * 32, 0);
-      R.b0w = v[0];
-      R.b1w = v[1];
-      R.b2w = v[2];
-      R.b3w = v[3];
+      R.bw = __builtin_amdgcn_raw_buffer_load_b128(wr, w_voff, ks * 32, 0);
     }
-    R.sreg = __builtin_amdgcn_raw_buffer_load_b16(sr, g_voff, (ks >> 1) * 2, 0);
-    R.bireg = __builtin_amdgcn_raw_buffer_load_b16(brs, g_voff, (ks >> 1) * 2, 0);
   };
 
   // ---- register -> LDS stage: copy A, dequantise B once for the whole block
-  auto stage = [&](int buf, const Stage &R) __attribute__((always_inline)) {
-    As[buf][tile_off(arg, acp)] = R.a0;
-    As[buf][tile_off(arg + 64, acp)] = R.a1;
-    As[buf][tile_off(arg + 128, acp)] = R.a2;
-    As[buf][tile_off(arg + 192, acp)] = R.a3;
-    const float sc = bf16lo_to_f32(R.sreg);
-    float bi = bf16lo_to_f32(R.bireg);
+  auto stage = [&](int buf, const Stage &R, const SbWindow &sb, int step) __attribute__((always_inline)) {
+    u32x4_t *const At = As(buf), *const Bt = Bs(buf);
+    At[tile_off(arg, acp)] = R.a0;
+    At[tile_off(arg + 128, acp)] = R.a1;
+    // group of this step inside the window: which thread of the row holds it, which word, which half
+    const int gi = (step >> 1) & 7;
+    uint32_t sw = (gi & 2) ? sb.s[1] : sb.s[0];
+    uint32_t bw = (gi & 2) ? sb.b[1] : sb.b[0];
+    const uint32_t sn = (uint32_t)__builtin_amdgcn_mov_dpp((int)sw, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+    const uint32_t bn = (uint32_t)__builtin_amdgcn_mov_dpp((int)bw, 0xB1, 0xf, 0xf, true);
+    if ((gi >> 2) != bh) {
+      sw = sn;
+      bw = bn;
+    }
+    const float sc = (gi & 1) ? bf16hi_to_f32(sw) : bf16lo_to_f32(sw);
+    float bi = (gi & 1) ? bf16hi_to_f32(bw) : bf16lo_to_f32(bw);
     if constexpr (BITS == 4) {
       bi = __builtin_fmaf(-128.0f, sc, bi);  // codes are expanded as 128 + q
 #pragma unroll
       for (int wi = 0; wi < 2; ++wi) {
-        const uint32_t w = wi == 0 ? R.b0w : R.b1w;
+        const uint32_t w = R.bw[wi];
         uint32_t o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t pr = ((w >> (4 * i)) & 0x000f000fu) | 0x43004300u;  // (128+q_i, 128+q_{i+4})
           o[i] = cvt_pk_bf16(__builtin_fmaf(sc, bf16lo_to_f32(pr), bi), __builtin_fmaf(sc, bf16hi_to_f32(pr), bi));
         }
-        Bs[buf][tile_off(br, 2 * bh + wi)] = u32x4_t{o[0], o[1], o[2], o[3]};
+        Bt[tile_off(br, 2 * bh + wi)] = u32x4_t{o[0], o[1], o[2], o[3]};
       }
     } else {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {  // 8 codes = two words -> one chunk
-        const uint32_t wA = h == 0 ? R.b0w : R.b2w, wB = h == 0 ? R.b1w : R.b3w;
+        const uint32_t wA = R.bw[2 * h], wB = R.bw[2 * h + 1];
         uint32_t o[4];
         o[0] = cvt_pk_bf16(__builtin_fmaf(sc, (float)(wA & 0xffu), bi), __builtin_fmaf(sc, (float)((wA >> 8) & 0xffu), bi));
         o[1] = cvt_pk_bf16(__builtin_fmaf(sc, (float)((wA >> 16) & 0xffu), bi), __builtin_fmaf(sc, (float)(wA >> 24), bi));
         o[2] = cvt_pk_bf16(__builtin_fmaf(sc, (float)(wB & 0xffu), bi), __builtin_fmaf(sc, (float)((wB >> 8) & 0xffu), bi));
         o[3] = cvt_pk_bf16(__builtin_fmaf(sc, (float)((wB >> 16) & 0xffu), bi), __builtin_fmaf(sc, (float)(wB >> 24), bi));
-        Bs[buf][tile_off(br, 2 * bh + h)] = u32x4_t{o[0], o[1], o[2], o[3]};
+        Bt[tile_off(br, 2 * bh + h)] = u32x4_t{o[0], o[1], o[2], o[3]};
       }
     }
   };
@@ -164,44 +196,80 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[m][s][r] = 0.f;
   const int ln = lane & 31, kb = lane >> 5;
-  const int brow0 = (GLU ? 32 * wn : 64 * wn) + ln;            // gate rows / first 32 rows
-  const int brow1 = (GLU ? 64 + 32 * wn : 64 * wn + 32) + ln;  // the matching up rows / next 32
+  const int brow0 = (GLU ? 32 * wn : 64 * wn) + ln;             // gate rows / first 32 rows
+  const int brow1 = (GLU ? 128 + 32 * wn : 64 * wn + 32) + ln;  // the matching up rows / next 32
   const int arow0 = 128 * wm + ln;
 
   auto mma = [&](int cur) __attribute__((always_inline)) {
+    const u32x4_t *const At = As(cur), *const Bt = Bs(cur);
 #pragma unroll
     for (int ss = 0; ss < 2; ++ss) {
       const int c = 2 * kb + ss;
-      const u32x4_t b0 = Bs[cur][tile_off(brow0, c)];
-      const u32x4_t b1 = Bs[cur][tile_off(brow1, c)];
+      const u32x4_t b0 = Bt[tile_off(brow0, c)];
+      const u32x4_t b1 = Bt[tile_off(brow1, c)];
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        const u32x4_t av = As[cur][tile_off(arow0 + 32 * m, c)];
+        const u32x4_t av = At[tile_off(arow0 + 32 * m, c)];
         acc[m][0] = mfma32(av, b0, acc[m][0]);
         acc[m][1] = mfma32(av, b1, acc[m][1]);
       }
     }
   };
 
-  // K loop, two steps per trip (nk is even: K is a multiple of 64).  Entering step ks: LDS buffer
-  // ks & 1 holds step ks, register set R1/R0 holds step ks + 1, the load of step ks + 2 is in flight.
+  // K loop.  nk is a multiple of 4 (the launcher takes K in multiples of 128 only).  Step ks:
+  // stage step ks from register set ks & 3 into LDS buffer ks & 1 (last read two steps ago, before
+  // the previous barrier), reload the set freed one step ago with step ks + 3, multiply step ks - 1
+  // from the other buffer.  Steps ks + 1 .. ks + 3 are in flight meanwhile.  Outer loop: one window
+  // of scales / biases (16 steps), whose loads sit outside any condition for the same reason the
+  // step loads do, and which is only read in the iteration after the one that loaded it.
   const int nk = K / BK;
-  Stage R0, R1;
-  gload(0, R0);
-  gload(1, R1);
-  stage(0, R0);
-  if (nk > 2) gload(2, R0);
-  __syncthreads();
-  for (int ks = 0; ks < nk; ks += 2) {
-    stage(1, R1);                          // step ks + 1 -> buffer 1 (last read before the previous barrier)
-    if (ks + 3 < nk) gload(ks + 3, R1);
-    mma(0);                                // step ks
-    __syncthreads();
-    if (ks + 2 < nk) stage(0, R0);         // step ks + 2 -> buffer 0
-    if (ks + 4 < nk) gload(ks + 4, R0);
-    mma(1);                                // step ks + 1
-    __syncthreads();
+  Stage R[DEPTH];
+  SbWindow sb_cur, sb_next = load_window(0);
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d) gload(d, R[d]);
+
+  // four steps, register sets and LDS buffers by constant index.  FIRST: steps 0..3, where step 0
+  // has nothing to multiply yet.  Inside a step the dequantisation arithmetic of the stage is
+  // independent of the MFMAs (they work on the other LDS buffer), and the two waves of a SIMD run
+  // their steps in phase (same block, same barriers), so the scheduler is asked to weave the
+  // stage's VALU work between the MFMAs instead of running the two phases one after the other.
+  auto group = [&](int kq, auto first) __attribute__((always_inline)) {
+    constexpr bool FIRST = decltype(first)::value;
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int ks = kq + d;
+      gload(ks + DEPTH - 1 < nk ? ks + DEPTH - 1 : nk - 1, R[(d + DEPTH - 1) & 3]);  // a repeat at the very end
+      // the multiply comes first in program order: its LDS reads must not queue behind the stage's
+      // LDS writes (the compiler cannot tell the two buffers apart), which hang on the stage's VALU work
+      if (!(FIRST && d == 0)) mma((d + 1) & 1);
+      stage(d & 1, R[d], sb_cur, ks);
+#if MI_MOE_WEAVE
+      if (!(FIRST && d == 0)) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);  // first operands from LDS
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // four VALU of the stage
+          if (i < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the remaining LDS reads
+        }
+      }
+#endif
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);  // nothing moves between steps: a stage hoisted across would
+                                          // wait for its loads one step early
+    }
+  };
+  sb_cur = sb_next;
+  sb_next = load_window(1);
+  group(0, std::true_type{});
+  for (int kq = DEPTH; kq < (16 < nk ? 16 : nk); kq += DEPTH) group(kq, std::false_type{});
+  for (int k0 = 16; k0 < nk; k0 += 16) {
+    sb_cur = sb_next;
+    sb_next = load_window((k0 >> 4) + 1);
+    const int k1 = k0 + 16 < nk ? k0 + 16 : nk;
+    for (int kq = k0; kq < k1; kq += DEPTH) group(kq, std::false_type{});
   }
+  mma(1);  // step nk - 1 (odd)
 
   // ---- epilogue: D[i][j], lane holds column j = lane % 32 and rows 8 (r/4) + 4 (lane/32) + r%4.
   // perm_out: columns are written in the paired order within each 8-block (what a 4-bit
@@ -260,15 +328,26 @@ hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *ou
 
 hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
   if (!a.mtiles || a.max_mtiles <= 0 || !a.x_perm) return hipSuccess;
-  const int ni = glu ? 64 : 128;
+  const int ni = glu ? 128 : 256;
   const int n_ntiles = (a.N + ni - 1) / ni;
   const unsigned grid = (unsigned)((a.max_mtiles + 7) / 8) * 8u * (unsigned)n_ntiles;
+  // 80 KB of LDS per block: above the 64 KB a kernel gets without asking
+  static bool lds_raised = false;
+  if (!lds_raised) {
+    const int bytes = (int)kLargeLdsBytes;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<4, true>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<4, false>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<8, true>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<8, false>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return e;
+    lds_raised = true;
+  }
   if (a.bits == 4) {
-    if (glu) qmm_large_kernel<4, true><<<grid, 256, 0, st>>>(a, n_ntiles);
-    else qmm_large_kernel<4, false><<<grid, 256, 0, st>>>(a, n_ntiles);
+    if (glu) qmm_large_kernel<4, true><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
+    else qmm_large_kernel<4, false><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
   } else {
-    if (glu) qmm_large_kernel<8, true><<<grid, 256, 0, st>>>(a, n_ntiles);
-    else qmm_large_kernel<8, false><<<grid, 256, 0, st>>>(a, n_ntiles);
+    if (glu) qmm_large_kernel<8, true><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
+    else qmm_large_kernel<8, false><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
   }
   return hipGetLastError();
 }

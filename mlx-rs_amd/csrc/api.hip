@@ -86,6 +86,7 @@ struct ForwardWs {
   uint16_t *topk_w;
   uint32_t *counts, *offsets, *work, *mtiles, *perm, *inv_perm, *src_of;
   int max_mtiles;
+  bool tiled;
   void *disp_scratch;
   uint16_t *hh, *y, *xperm;
   size_t bytes;
@@ -101,20 +102,21 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.counts = cv.take<uint32_t>(c.n_experts);
   f.offsets = cv.take<uint32_t>(c.n_experts + 1);
   f.work = cv.take<uint32_t>((size_t)c.n_experts * 16);
-  // M tiles of the tiled kernel: at most one partial tile per long segment plus P / tile full ones
-  // (a segment is at most T rows long: no token picks an expert twice)
+  // M tiles of the tiled kernel: the 256-row list holds at most P / 256 full tiles plus one
+  // remainder per tiled segment (a segment is at most T rows long: no token picks an expert twice)
   // (the tiled kernel reads scales in 8-byte pieces: rows of scales must be 4-byte aligned, i.e.
   // an even number of groups per row; other shapes stay on the streaming kernel)
   const bool tiled_ok = (c.hidden / 64) % 2 == 0 && (c.intermediate / 64) % 2 == 0;
-  f.max_mtiles = T >= kBigThreshold && tiled_ok ? (int)(P / kBigTileM + (P / kBigThreshold < c.n_experts ? P / kBigThreshold : c.n_experts)) : 0;
-  f.mtiles = cv.take<uint32_t>(4 + (size_t)f.max_mtiles * 4);
+  f.tiled = T >= kTiledMinTokens && tiled_ok;
+  f.max_mtiles = f.tiled ? (int)(P / kBigTileM + (P / kTileMinRows < c.n_experts ? P / kTileMinRows : c.n_experts)) : 0;
+  f.mtiles = cv.take<uint32_t>(tile_list_words(f.max_mtiles, c.n_experts));
   f.perm = cv.take<uint32_t>((size_t)P);
   f.inv_perm = cv.take<uint32_t>((size_t)P);
   f.src_of = cv.take<uint32_t>((size_t)P);
   f.disp_scratch = cv.take<char>(dispatch_workspace_bytes(c.n_experts, P));
   f.hh = cv.take<uint16_t>((size_t)P * c.intermediate);
   f.y = cv.take<uint16_t>((size_t)P * c.hidden);
-  f.xperm = cv.take<uint16_t>(f.max_mtiles && c.bits == 4 ? (size_t)T * c.hidden : 0);
+  f.xperm = cv.take<uint16_t>(f.tiled && c.bits == 4 ? (size_t)T * c.hidden : 0);
   f.bytes = cv.off;
   return f;
 }
@@ -210,8 +212,8 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
     // decode: one launch for the three stages (the stage times then all land in the first)
     MI_HIP(launch_router_fused(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, c.top_k,
                                c.score_mode, f.logits, f.topk_idx, f.topk_w, h->counters, f.counts, f.offsets,
-                               f.perm, f.inv_perm, f.src_of, f.work, f.max_mtiles ? f.mtiles : nullptr,
-                               kBigThreshold, st));
+                               f.perm, f.inv_perm, f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles,
+                               kTileMinRows, st));
     MI_STAGE_DONE();
     MI_STAGE_DONE();
     MI_STAGE_DONE();
@@ -221,25 +223,27 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
     MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
     MI_STAGE_DONE();
     MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
-                           f.src_of, f.work, f.max_mtiles ? f.mtiles : nullptr, kBigThreshold, f.disp_scratch, st));
+                           f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles, kTileMinRows,
+                           f.disp_scratch, st));
     MI_STAGE_DONE();
   }
   const int max_active = (int)(P < c.n_experts ? P : c.n_experts);
   GroupedArgs a{};
   a.work = f.work;
   a.max_active = max_active;
-  a.mtiles = f.max_mtiles ? f.mtiles : nullptr;
+  a.mtiles = f.tiled ? f.mtiles : nullptr;
   a.max_mtiles = f.max_mtiles;
+  a.tile_cap_e = f.tiled ? c.n_experts : 0;
   a.bits = c.bits;
   a.total_rows = P;
   a.max_rows_per_expert = T;  // a token picks an expert at most once
   // 4-bit: the tiled kernel reads activations with paired 8-blocks; h is produced that way,
   // x is copied once per forward (prefill-sized T only)
   const bool paired = c.bits == 4;
-  if (f.max_mtiles && paired) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
+  if (f.tiled && paired) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
   // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
   a.x = x;
-  a.x_perm = paired ? (f.max_mtiles ? f.xperm : nullptr) : x;
+  a.x_perm = paired ? (f.tiled ? f.xperm : nullptr) : x;
   a.x_paired = false;
   a.y_paired = paired;
   a.src_rows = f.src_of;
@@ -362,7 +366,7 @@ int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts
   void *scratch = cv.take<char>(dispatch_workspace_bytes(n_experts, P));
   hipStream_t st = static_cast<hipStream_t>(stream);
   MI_HIP(launch_dispatch(expert_of_pair, P, n_experts, 1, counts, offsets, perm, inv_perm, nullptr, nullptr,
-                         nullptr, 0, scratch, st));
+                         nullptr, 0, 0, scratch, st));
   return 0;
 }
 
@@ -410,7 +414,7 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   uint32_t *dst_rows = cv.take<uint32_t>((size_t)rows);
   hipStream_t st = static_cast<hipStream_t>(stream);
   MI_HIP(launch_dispatch(rhs_indices, n_idx, n_experts, 1, counts, offsets, perm, nullptr, nullptr, work,
-                         nullptr, 0, scratch, st));
+                         nullptr, 0, 0, scratch, st));
   MI_HIP(launch_row_maps(perm, lhs_indices, offsets, n_idx, M, n_experts, src_rows, dst_rows, work, st));
   GroupedArgs a{};
   a.x = x;
@@ -431,9 +435,9 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
 
 static size_t qmm_dense_bytes(int64_t M, int32_t K, int32_t bits, size_t *mt_words) {
   const size_t ntiles = (size_t)((M + kBigTileM - 1) / kBigTileM);
-  *mt_words = 4 + 4 * ntiles;
+  *mt_words = tile_list_words((int)ntiles, 1);
   size_t b = 256 + 64 + *mt_words * 4 + 256;
-  if (bits == 4 && M >= kBigThreshold) b += (size_t)M * K * 2 + 256;
+  if (bits == 4 && M >= kTileMinRows) b += (size_t)M * K * 2 + 256;
   return b;
 }
 
@@ -466,10 +470,11 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
   Carver cv(workspace);
   uint32_t *work = cv.take<uint32_t>(16);
   uint32_t *mtiles = cv.take<uint32_t>(mt_words);
-  const bool big = M >= kBigThreshold && (K / 64) % 2 == 0;
+  const bool big = M >= kTileMinRows && (K / 64) % 2 == 0;
   uint16_t *xperm = (bits == 4 && big) ? cv.take<uint16_t>((size_t)M * K) : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  MI_HIP(launch_dense_records(M, big ? kBigThreshold : 0, work, mtiles, st));
+  const int cap256 = (int)((M + kBigTileM - 1) / kBigTileM);
+  MI_HIP(launch_dense_records(M, big ? kTileMinRows : 0, work, mtiles, cap256, st));
   if (xperm) MI_HIP(launch_pair_rows(x, M, K, xperm, st));
   GroupedArgs a{};
   a.x = x;
@@ -477,7 +482,8 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
   a.work = work;
   a.max_active = 1;
   a.mtiles = big ? mtiles : nullptr;
-  a.max_mtiles = big ? (int)((M + kBigTileM - 1) / kBigTileM) : 0;
+  a.max_mtiles = big ? cap256 : 0;
+  a.tile_cap_e = big ? 1 : 0;
   a.w0 = w; a.s0 = scales; a.b0 = biases;
   a.y = y;
   a.N = N;

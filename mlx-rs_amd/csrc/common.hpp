@@ -7,8 +7,9 @@
 namespace mi_moe {
 
 constexpr int kWave = 64;
-constexpr int kBigThreshold = 48;  // segments with at least this many rows use the tiled kernel
-constexpr int kBigTileM = 256;     // rows per M tile of the tiled kernel
+constexpr int kTiledMinTokens = 192; // batches from this size on cut their longer segments into M tiles
+constexpr int kTileMinRows = 9;      // ... the segments of at least this many rows (up to 8: one pass of the streaming kernel)
+constexpr int kBigTileM = 256;       // rows of the largest M tile
 constexpr int kFusedRouterMaxTokens = 64;  // up to here router + dispatch run as one launch
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
@@ -86,6 +87,22 @@ __device__ __forceinline__ float wave_max_f32(float v) {
   return v;
 }
 
+// ---------------------------------------------------------------- M-tile lists
+// Three lists, for tiles of 256, 128 and 64 rows, back to back in one buffer: a segment of at least
+// kTileMinRows rows is cut into 256-row tiles; what is left goes to the smallest class that holds
+// it.  List layout: word 0 = number of tiles, tile i at words 4 + 4 i = {expert, first sorted row,
+// rows, 0}.  Capacities: cap256 for the first list, n_experts for the other two (a segment leaves
+// at most one remainder).
+__host__ __device__ inline size_t tile_list_words(int cap256, int n_experts) {
+  return (4 + 4 * (size_t)cap256) + 2 * (4 + 4 * (size_t)n_experts);
+}
+template <class P>
+__host__ __device__ inline P *tile_list(P *base, int cls, int cap256, int n_experts) {
+  if (cls == 0) return base;
+  if (cls == 1) return base + 4 + 4 * (size_t)cap256;
+  return base + 4 + 4 * (size_t)cap256 + 4 + 4 * (size_t)n_experts;
+}
+
 // ---------------------------------------------------------------- device-coherent accesses
 // A load that observes what other workgroups have written before an agent-scope release
 // (bypasses the per-CU cache).  Used for data produced earlier in the same launch.
@@ -112,8 +129,9 @@ struct GroupedArgs {
   const uint32_t *dst_rows; // output row of sorted row r, or nullptr = r
   const uint32_t *work;        // 16-word records {expert, first row, rows, has_src, src[12]}, count 0 = end
   int max_active;              // upper bound of the number of records known on the host
-  const uint32_t *mtiles;      // M tiles of the long segments (tiled MFMA kernel), or nullptr
-  int max_mtiles;              // host upper bound of the number of M tiles
+  const uint32_t *mtiles;      // M-tile lists (tiled MFMA kernel), or nullptr
+  int max_mtiles;              // capacity of the 256-row list
+  int tile_cap_e;              // capacity of the 128- and 64-row lists (the number of experts)
   const uint32_t *w0, *w1;     // packed weights [E,N,K*bits/32]; w1 only for GLU
   const uint16_t *s0, *b0, *s1, *b1;
   uint16_t *y;                 // bf16 [rows, N]
@@ -129,7 +147,7 @@ hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k,
 size_t dispatch_workspace_bytes(int E, int64_t P);
 hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
                            uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                           uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
+                           uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int cap256, int big_thr,
                            void *scratch, hipStream_t st);
 // decode-sized batches: logits + selection + dispatch in one launch.  counters: 1 +
 // kFusedRouterMaxTokens zero-initialised words that the kernel leaves zeroed again.
@@ -138,15 +156,16 @@ hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const floa
                                int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx,
                                uint16_t *topk_w, uint32_t *counters, uint32_t *counts,
                                uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                               uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
-                               hipStream_t st);
+                               uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int cap256,
+                               int big_thr, hipStream_t st);
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *out, hipStream_t st);
 hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
                            uint32_t *work, hipStream_t st);
-hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t *mtiles, hipStream_t st);
+hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t *mtiles, int cap256,
+                                hipStream_t st);
 hipError_t launch_swiglu(const uint16_t *g, const uint16_t *u, int64_t n, uint16_t *out,
                          hipStream_t st);
 hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,

@@ -16,9 +16,9 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_single_kernel(
     const uint32_t *flat, int64_t P, int E, int nbits, int k_div,
     uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets, uint32_t *__restrict__ perm,
     uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of,
-    uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles, uint32_t big_thr) {
+    uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles, int cap256, uint32_t big_thr) {
   extern __shared__ uint32_t lds[];
-  dispatch_block(flat, P, E, nbits, k_div, lds, counts, offsets, perm, inv_perm, src_of, work, mtiles, big_thr);
+  dispatch_block(flat, P, E, nbits, k_div, lds, counts, offsets, perm, inv_perm, src_of, work, mtiles, cap256, big_thr);
 }
 
 // ---- three kernels for prefill-sized P: block b owns pairs [b*span, (b+1)*span)
@@ -42,7 +42,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(
 __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
     uint32_t *__restrict__ blockhist, int nb, int E, uint32_t *__restrict__ counts,
     uint32_t *__restrict__ offsets, uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
-    uint32_t big_thr) {
+    int cap256, uint32_t big_thr) {
   extern __shared__ uint32_t lds[];
   __shared__ uint32_t n_active;
   uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
     cnt[tid] = run;
   }
   __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, big_thr, &n_active);
+  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, cap256, big_thr, &n_active);
   if (tid < E) {  // blockhist[b][e] <- first sorted position of expert e for block b
     uint32_t run = cur[tid];
     for (int b = 0; b < nb; ++b) {
@@ -88,7 +88,7 @@ size_t dispatch_workspace_bytes(int E, int64_t P) {
 
 hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, uint32_t *counts,
                            uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                           uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
+                           uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int cap256, int big_thr,
                            void *scratch, hipStream_t st) {
   int nbits = 0;
   while ((1 << nbits) < E) ++nbits;
@@ -96,29 +96,41 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
   if (P <= kSingleMaxP) {
     size_t lds = (size_t)(3 + kDispWaves) * E * sizeof(uint32_t);
     dispatch_single_kernel<<<1, kDispThreads, lds, st>>>(flat, P, E, nbits, k_div, counts, offsets,
-                                                        perm, inv_perm, src_of, work, mtiles, (uint32_t)big_thr);
+                                                        perm, inv_perm, src_of, work, mtiles, cap256, (uint32_t)big_thr);
     return hipGetLastError();
   }
   uint32_t *blockhist = reinterpret_cast<uint32_t *>(scratch);
   const int nb = (int)((P + kSpan - 1) / kSpan);
   dispatch_hist_kernel<<<nb, kDispThreads, (size_t)E * 4, st>>>(flat, P, E, kSpan, blockhist);
   dispatch_scan_kernel<<<1, kDispThreads, (size_t)3 * E * 4, st>>>(blockhist, nb, E, counts,
-                                                                  offsets, work, mtiles, (uint32_t)big_thr);
+                                                                  offsets, work, mtiles, cap256, (uint32_t)big_thr);
   dispatch_scatter_kernel<<<nb, kDispThreads, (size_t)(1 + kDispWaves) * E * 4, st>>>(
       flat, P, E, nbits, k_div, kSpan, blockhist, perm, inv_perm, src_of);
   return hipGetLastError();
 }
 
 // One dense segment (a plain quantized matmul: every row goes to matrix 0): the work record or, from
-// big_thr rows on, the M tiles of the tiled kernel.
+// big_thr rows on, its M tiles.
 __global__ void dense_records_kernel(uint32_t M, uint32_t big_thr, uint32_t *__restrict__ work,
-                                     uint32_t *__restrict__ mtiles) {
+                                     uint32_t *__restrict__ mtiles, int cap256) {
   const uint32_t tid = threadIdx.x;
   const bool big = big_thr != 0u && M >= big_thr;
-  const uint32_t ntiles = big ? (M + kBigTileM - 1) / kBigTileM : 0u;
   if (tid < kWorkWords) work[tid] = (tid == 2 && !big) ? M : 0u;  // {expert 0, row 0, M rows, no inline rows}
-  if (tid == 0) mtiles[0] = ntiles;
-  for (uint32_t i = tid; i < ntiles; i += blockDim.x) {
+  const TileSplit ts = split_segment(big ? M : 0u);
+  uint32_t *const l128 = tile_list(mtiles, 1, cap256, 1), *const l64 = tile_list(mtiles, 2, cap256, 1);
+  if (tid == 0) {
+    mtiles[0] = ts.n256;
+    l128[0] = big && ts.r != 0u && ts.rcls == 1;
+    l64[0] = big && ts.r != 0u && ts.rcls == 2;
+    if (big && ts.r != 0u && ts.rcls != 0) {
+      uint32_t *rec = (ts.rcls == 1 ? l128 : l64) + 4;
+      rec[0] = 0u;
+      rec[1] = M - ts.r;
+      rec[2] = ts.r;
+      rec[3] = 0u;
+    }
+  }
+  for (uint32_t i = tid; i < ts.n256; i += blockDim.x) {
     uint32_t *rec = mtiles + 4 + (size_t)i * 4;
     rec[0] = 0u;
     rec[1] = i * kBigTileM;
@@ -127,8 +139,9 @@ __global__ void dense_records_kernel(uint32_t M, uint32_t big_thr, uint32_t *__r
   }
 }
 
-hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t *mtiles, hipStream_t st) {
-  dense_records_kernel<<<1, 256, 0, st>>>((uint32_t)M, (uint32_t)big_thr, work, mtiles);
+hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t *mtiles, int cap256,
+                                hipStream_t st) {
+  dense_records_kernel<<<1, 256, 0, st>>>((uint32_t)M, (uint32_t)big_thr, work, mtiles, cap256);
   return hipGetLastError();
 }
 

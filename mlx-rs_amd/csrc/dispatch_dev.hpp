@@ -92,15 +92,29 @@ __device__ __forceinline__ void scatter_range(const uint32_t *flat, int64_t j0, 
 constexpr int kWorkWords = 16;
 constexpr int kWorkSrc = 12;
 
-// Long segments (at least big_thr rows, big_thr > 0) go to the tiled MFMA kernel instead: they
-// are cut into M tiles of kBigTileM rows, listed in `mtiles`:
-//   mtiles[0] = number of tiles; tile i at mtiles[4 + 4 i] = {expert id, first sorted row, rows, 0}
+// Segments of at least big_thr rows (big_thr > 0) go to the tiled MFMA kernel instead: they are cut
+// into M tiles of 256 rows, and what is left over (or a whole shorter segment) goes to the smallest
+// of the 256-, 128- and 64-row classes that holds it; one list per class (tile_list()).
 
+// tile classes of a segment of c rows: full 256-row tiles, then one tile for the remainder r
+struct TileSplit {
+  uint32_t n256;  // tiles in the 256-row list (the last one may be the remainder, if r > 128)
+  uint32_t r;     // rows of the remainder tile (0: none)
+  int rcls;       // class of the remainder tile: 0, 1, 2
+};
+__device__ __forceinline__ TileSplit split_segment(uint32_t c) {
+  TileSplit t;
+  const uint32_t full = c / kBigTileM;
+  t.r = c % kBigTileM;
+  t.rcls = t.r > 128u ? 0 : (t.r > 64u ? 1 : 2);
+  t.n256 = full + (t.r > 128u ? 1u : 0u);
+  return t;
+}
 
 // counts -> offsets, work records and M tiles; runs in one block.  LDS cnt[E] in, cur[E] out.
 __device__ __forceinline__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint32_t *cur, int E,
                               uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
-                              uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
+                              uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles, int cap256,
                               uint32_t big_thr, uint32_t *n_active_lds) {
   __shared__ uint32_t total;
   const int tid = threadIdx.x;
@@ -115,7 +129,9 @@ __device__ __forceinline__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint
   __syncthreads();
   // experts with rows, in ascending order, by wave 0
   if (tid < kWave) {
-    uint32_t base = 0, tbase = 0;
+    uint32_t *const l256 = mtiles, *const l128 = mtiles ? tile_list(mtiles, 1, cap256, E) : nullptr,
+                   *const l64 = mtiles ? tile_list(mtiles, 2, cap256, E) : nullptr;
+    uint32_t base = 0, t256 = 0, t128 = 0, t64 = 0;
     for (int e0 = 0; e0 < E; e0 += kWave) {
       const int e = e0 + tid;
       uint32_t c = 0;
@@ -131,21 +147,35 @@ __device__ __forceinline__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint
         rec[3] = 0u;
       }
       base += __popcll(bm);
-      // M tiles of the long segments: exclusive scan of the tile counts over the wave
-      const uint32_t nt = big ? (c + kBigTileM - 1) / kBigTileM : 0u;
-      uint32_t incl = nt;
+      // M tiles: exclusive scan of the 256-row tile counts over the wave, ballots for the others
+      TileSplit ts = split_segment(big ? c : 0u);
+      uint32_t incl = ts.n256;
       for (int d = 1; d < kWave; d <<= 1) {
         const uint32_t v = __shfl_up(incl, d, kWave);
         if (tid >= d) incl += v;
       }
-      for (uint32_t i = 0; i < nt; ++i) {
-        uint32_t *rec = mtiles + 4 + (size_t)(tbase + incl - nt + i) * 4;
+      const uint32_t first = big ? cnt[e] : 0u;
+      for (uint32_t i = 0; i < ts.n256; ++i) {
+        uint32_t *rec = l256 + 4 + (size_t)(t256 + incl - ts.n256 + i) * 4;
+        const uint32_t left = c - i * kBigTileM;
         rec[0] = (uint32_t)e;
-        rec[1] = cnt[e] + i * kBigTileM;
-        rec[2] = c - i * kBigTileM < (uint32_t)kBigTileM ? c - i * kBigTileM : (uint32_t)kBigTileM;
+        rec[1] = first + i * kBigTileM;
+        rec[2] = left < (uint32_t)kBigTileM ? left : (uint32_t)kBigTileM;
         rec[3] = 0u;
       }
-      tbase += __shfl(incl, kWave - 1, kWave);
+      t256 += __shfl(incl, kWave - 1, kWave);
+      const bool r128 = big && ts.r != 0u && ts.rcls == 1, r64 = big && ts.r != 0u && ts.rcls == 2;
+      const uint64_t b128 = __ballot(r128), b64 = __ballot(r64);
+      if (r128 || r64) {
+        uint32_t *rec = r128 ? l128 + 4 + (size_t)(t128 + __popcll(b128 & lanemask_lt())) * 4
+                             : l64 + 4 + (size_t)(t64 + __popcll(b64 & lanemask_lt())) * 4;
+        rec[0] = (uint32_t)e;
+        rec[1] = first + (c - ts.r);
+        rec[2] = ts.r;
+        rec[3] = 0u;
+      }
+      t128 += __popcll(b128);
+      t64 += __popcll(b64);
     }
     if (work)
       for (int sl = base + tid; sl < E; sl += kWave) {
@@ -154,7 +184,11 @@ __device__ __forceinline__ void finish_counts(uint32_t *cnt, uint32_t *tmp, uint
       }
     if (tid == 0) {
       *n_active_lds = base;
-      if (mtiles) mtiles[0] = tbase;
+      if (mtiles) {
+        l256[0] = t256;
+        l128[0] = t128;
+        l64[0] = t64;
+      }
     }
   }
   __syncthreads();
@@ -167,7 +201,7 @@ __device__ __forceinline__ void dispatch_block(const uint32_t *flat, int64_t P, 
                                uint32_t *lds, uint32_t *__restrict__ counts,
                                uint32_t *__restrict__ offsets, uint32_t *__restrict__ perm,
                                uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of,
-                               uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
+                               uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles, int cap256,
                                uint32_t big_thr) {
   __shared__ uint32_t n_active;
   uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *wcnt = lds + 3 * E;
@@ -179,7 +213,7 @@ __device__ __forceinline__ void dispatch_block(const uint32_t *flat, int64_t P, 
     atomicAdd(&cnt[e < (uint32_t)E ? e : (uint32_t)E - 1u], 1u);
   }
   __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, big_thr, &n_active);
+  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, cap256, big_thr, &n_active);
   scatter_range(flat, 0, P, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
   // source rows of the first rows of every segment, so that a consumer needs one load
   if (work) {

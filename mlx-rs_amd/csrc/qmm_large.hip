@@ -1,9 +1,9 @@
-// Tiled grouped quantized product for long expert segments (prefill).
+// Tiled grouped quantized product for expert segments of more than 8 rows (prefill).
 //
 // Same contract as the small-segment kernel (mlx_gather_qmm with transpose = true,
 // mlx-rs/src/ops/quantization.rs:160-230; with GLU also nn::silu and multiply,
 // nn/activation.rs:142-144,876-880), restricted to the segments the dispatch cut into M tiles
-// of 256 rows.  A block of 8 waves computes a 256-token x 256-weight-row tile:
+// of 256, 128 or 64 rows.  A block of 8 waves computes a (256 | 128 | 64)-token x 256-weight-row tile:
 //   * weights stream from HBM as packed codes (one 8- or 16-byte load per thread and K step; scales
 //     and biases in 8-byte pieces that last 16 K steps),
 //     are dequantised ONCE per block to bf16 (w_hat = s q + b, fp32 fma, one rounding) and
@@ -27,7 +27,6 @@ namespace mi_moe {
 
 namespace {
 
-constexpr int BM = kBigTileM;  // token rows per block
 constexpr int BK = 32;         // K step (two steps per quantisation group)
 constexpr int BR = 256;        // weight rows per block (GLU: 128 gate + 128 up)
 constexpr int NTHREADS = 512;  // 8 waves: 2 (token halves) x 4 (weight-row quarters)
@@ -50,7 +49,7 @@ __device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
 // consecutive rows clear of each other.
 constexpr int LDR = 5;  // row stride in uint4 units
 __device__ __forceinline__ int tile_off(int row, int chunk) { return row * LDR + chunk; }
-constexpr size_t kLargeLdsBytes = (size_t)2 * (BM + BR) * LDR * 16;  // two steps of A and B tiles
+constexpr size_t large_lds_bytes(int bm) { return (size_t)2 * (bm + BR) * LDR * 16; }  // two steps of A and B tiles
 
 }  // namespace
 
@@ -61,18 +60,26 @@ constexpr size_t kLargeLdsBytes = (size_t)2 * (BM + BR) * LDR * 16;  // two step
 // thread needs per step, and the registers saved pay for four stages, i.e. three steps of loads in
 // flight.  Per-step 2-byte gathers of scales and biases (more expensive than all other loads of
 // that kernel together) became one 8-byte load per 16 steps.
-template <int BITS, bool GLU>
-__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void qmm_large_kernel(GroupedArgs a, int n_ntiles) {
+//
+// MT = token rows per block / 64 (4, 2 or 1): the same kernel on 256-, 128- and 64-row M tiles, so
+// that a short segment or the short end of a long one does not pay for 256 rows of MFMA work.  The
+// weight side (256 rows dequantised per step) is the same for all three; with 64 rows the kernel is
+// bound by that dequantisation, which is still far cheaper than streaming the weights once per
+// 8 tokens.
+template <int BITS, bool GLU, int MT>
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT == 4 ? 2 : 4))) void qmm_large_kernel(GroupedArgs a, const uint32_t *__restrict__ tiles, int n_ntiles) {
   constexpr int NI = GLU ? 128 : 256;  // distinct output columns per block
+  constexpr int BM = 64 * MT;          // token rows per block
+  constexpr int NA = MT >= 2 ? MT / 2 : 1;  // 16-byte activation loads per thread and step
 
   // block -> (M tile, N tile): blocks of one M tile share the gathered token rows, so they
   // are given consecutive ids on ONE XCD (ids are dealt round-robin over the 8 XCDs)
-  const uint32_t n_mtiles = a.mtiles[0];
+  const uint32_t n_mtiles = tiles[0];
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int nt = j % n_ntiles;
   const uint32_t mt_id = (uint32_t)(j / n_ntiles) * 8u + xcd;
   if (mt_id >= n_mtiles) return;
-  const uint4 rec = reinterpret_cast<const uint4 *>(a.mtiles)[1 + mt_id];
+  const uint4 rec = reinterpret_cast<const uint4 *>(tiles)[1 + mt_id];
   const int e = (int)rec.x;
   const int64_t row0 = rec.y;
   const int rows = (int)rec.z;
@@ -93,15 +100,18 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   // ---- global -> register stage
   // A: the activations arrive with every 8-block already in the (x0,x4,x1,x5,x2,x6,x3,x7) order
   // of the nibble unpacking (4-bit), so a row chunk is copied as it is.  Thread: chunk acp of
-  // rows arg and arg + 128.
+  // rows arg, arg + 128 (64-row tiles: the first four waves only).
   const int acp = tid & 3, arg = tid >> 2;
+  const bool a_loader = MT >= 2 || wave < 4;  // wave-uniform
   auto a_row_ptr = [&](int tr) {
     tr = tr < rows ? tr : rows - 1;  // rows past the segment repeat its last row (never stored)
     const int64_t r = row0 + tr;
     const int64_t src = a.src_rows ? (int64_t)a.src_rows[r] : r;
     return a.x_perm + src * K + acp * 8;
   };
-  const uint16_t *const arow[2] = {a_row_ptr(arg), a_row_ptr(arg + 128)};
+  const uint16_t *arow[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) arow[i] = a_row_ptr(arg + 128 * i);
   // B: thread covers 16 codes (half a K step) of weight row br; waves 0-3 / 4-7 hold gate / up
   const int br = tid >> 1, bh = tid & 1;
   const int mat = GLU ? (wave >> 2) : 0;  // wave-uniform
@@ -126,14 +136,14 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   };
 
   struct Stage {
-    u32x4_t a0, a1;
+    u32x4_t av[NA];
     u32x4_t bw;  // 4-bit: two words used
   };
   // every load is unconditional (indices are clamped by the caller): the compiler can then count
   // the loads in flight and wait for exactly the stage it needs
   auto gload = [&](int ks, Stage &R) __attribute__((always_inline)) {
-    R.a0 = *reinterpret_cast<const u32x4_t *>(arow[0] + ks * BK);
-    R.a1 = *reinterpret_cast<const u32x4_t *>(arow[1] + ks * BK);
+#pragma unroll
+    for (int i = 0; i < NA; ++i) R.av[i] = *reinterpret_cast<const u32x4_t *>(arow[i] + ks * BK);
     if constexpr (BITS == 4) {
       const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(wr, w_voff, ks * 16, 0);
       R.bw[0] = v[0];
@@ -146,8 +156,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   // ---- register -> LDS stage: copy A, dequantise B once for the whole block
   auto stage = [&](int buf, const Stage &R, const SbWindow &sb, int step) __attribute__((always_inline)) {
     u32x4_t *const At = As(buf), *const Bt = Bs(buf);
-    At[tile_off(arg, acp)] = R.a0;
-    At[tile_off(arg + 128, acp)] = R.a1;
+    if (a_loader) {
+#pragma unroll
+      for (int i = 0; i < NA; ++i) At[tile_off(arg + 128 * i, acp)] = R.av[i];
+    }
     // group of this step inside the window: which thread of the row holds it, which word, which half
     const int gi = (step >> 1) & 7;
     uint32_t sw = (gi & 2) ? sb.s[1] : sb.s[0];
@@ -187,10 +199,12 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
   };
 
-  // ---- MFMA stage: wave (wm, wn) owns token rows [128 wm, +128) and two 32-row weight sub-tiles
-  f32x16_t acc[4][2];
+  // ---- MFMA stage: wave (wm, wn) owns token rows [BM/2 wm, + BM/2) and two 32-row weight
+  // sub-tiles.  64-row tiles: one 32-row sub-tile per wave.
+  constexpr int MS = MT >= 2 ? MT : 1;  // 32-row token sub-tiles per wave
+  f32x16_t acc[MS][2];
 #pragma unroll
-  for (int m = 0; m < 4; ++m)
+  for (int m = 0; m < MS; ++m)
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -198,7 +212,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int ln = lane & 31, kb = lane >> 5;
   const int brow0 = (GLU ? 32 * wn : 64 * wn) + ln;             // gate rows / first 32 rows
   const int brow1 = (GLU ? 128 + 32 * wn : 64 * wn + 32) + ln;  // the matching up rows / next 32
-  const int arow0 = 128 * wm + ln;
+  const int arow0 = (BM / 2) * wm + ln;
 
   auto mma = [&](int cur) __attribute__((always_inline)) {
     const u32x4_t *const At = As(cur), *const Bt = Bs(cur);
@@ -208,7 +222,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
       const u32x4_t b0 = Bt[tile_off(brow0, c)];
       const u32x4_t b1 = Bt[tile_off(brow1, c)];
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
+      for (int m = 0; m < MS; ++m) {
         const u32x4_t av = At[tile_off(arow0 + 32 * m, c)];
         acc[m][0] = mfma32(av, b0, acc[m][0]);
         acc[m][1] = mfma32(av, b1, acc[m][1]);
@@ -245,12 +259,12 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
       stage(d & 1, R[d], sb_cur, ks);
 #if MI_MOE_WEAVE
       if (!(FIRST && d == 0)) {
-        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);  // first operands from LDS
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 + MS, 0);  // first operands from LDS
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < 4 * MS; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // four VALU of the stage
-          if (i < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the remaining LDS reads
+          __builtin_amdgcn_sched_group_barrier(0x002, 16 / MS, 0);  // its share of the stage's VALU work
+          if (i < 2 + MS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the remaining LDS reads
         }
       }
 #endif
@@ -280,10 +294,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     return (col & ~7) | (jj < 4 ? 2 * jj : 2 * (jj - 4) + 1);
   };
 #pragma unroll
-  for (int m = 0; m < 4; ++m)
+  for (int m = 0; m < MS; ++m)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int tr = 128 * wm + 32 * m + 8 * (r >> 2) + 4 * kb + (r & 3);
+      const int tr = (BM / 2) * wm + 32 * m + 8 * (r >> 2) + 4 * kb + (r & 3);
       if (tr < rows) {
         const int64_t rr = row0 + tr;
         const int64_t dst = a.dst_rows ? (int64_t)a.dst_rows[rr] : rr;
@@ -326,30 +340,40 @@ hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *ou
   return hipGetLastError();
 }
 
-hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
-  if (!a.mtiles || a.max_mtiles <= 0 || !a.x_perm) return hipSuccess;
-  const int ni = glu ? 128 : 256;
+template <int BITS, bool GLU, int MT>
+static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int cap, hipStream_t st) {
+  const int ni = GLU ? 128 : 256;
   const int n_ntiles = (a.N + ni - 1) / ni;
-  const unsigned grid = (unsigned)((a.max_mtiles + 7) / 8) * 8u * (unsigned)n_ntiles;
-  // 80 KB of LDS per block: above the 64 KB a kernel gets without asking
-  static bool lds_raised = false;
-  if (!lds_raised) {
-    const int bytes = (int)kLargeLdsBytes;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<4, true>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<4, false>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<8, true>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<8, false>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e != hipSuccess) return e;
-    lds_raised = true;
+  const unsigned grid = (unsigned)((cap + 7) / 8) * 8u * (unsigned)n_ntiles;
+  constexpr size_t lds = large_lds_bytes(64 * MT);
+  // more LDS per block than a kernel gets without asking
+  static bool raised = false;
+  if (!raised) {
+    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<BITS, GLU, MT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e != hipSuccess)
+      return e;
+    raised = true;
   }
-  if (a.bits == 4) {
-    if (glu) qmm_large_kernel<4, true><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
-    else qmm_large_kernel<4, false><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
-  } else {
-    if (glu) qmm_large_kernel<8, true><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
-    else qmm_large_kernel<8, false><<<grid, NTHREADS, kLargeLdsBytes, st>>>(a, n_ntiles);
-  }
+  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles);
   return hipGetLastError();
+}
+
+template <int BITS, bool GLU>
+static hipError_t launch_classes(const GroupedArgs &a, hipStream_t st) {
+  // a segment is at most max_rows_per_expert long: classes that cannot occur are not launched
+  const int cap_small = a.tile_cap_e;
+  if (a.max_rows_per_expert > 128)
+    if (hipError_t e = launch_one<BITS, GLU, 4>(a, tile_list(a.mtiles, 0, a.max_mtiles, a.tile_cap_e), a.max_mtiles, st); e != hipSuccess) return e;
+  if (a.max_rows_per_expert > 64)
+    if (hipError_t e = launch_one<BITS, GLU, 2>(a, tile_list(a.mtiles, 1, a.max_mtiles, a.tile_cap_e), cap_small, st); e != hipSuccess) return e;
+  return launch_one<BITS, GLU, 1>(a, tile_list(a.mtiles, 2, a.max_mtiles, a.tile_cap_e), cap_small, st);
+}
+
+hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
+  if (!a.mtiles || a.tile_cap_e <= 0 || !a.x_perm) return hipSuccess;
+  if (a.bits == 4) return glu ? launch_classes<4, true>(a, st) : launch_classes<4, false>(a, st);
+  return glu ? launch_classes<8, true>(a, st) : launch_classes<8, false>(a, st);
 }
 
 }  // namespace mi_moe

@@ -25,7 +25,7 @@ __global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg, const float *__restrict__ bias,
     int T, int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx, uint16_t *topk_w,
     uint32_t *counters, int nbits, uint32_t *counts, uint32_t *offsets, uint32_t *perm,
-    uint32_t *inv_perm, uint32_t *src_of, uint32_t *work, uint32_t *mtiles, uint32_t big_thr) {
+    uint32_t *inv_perm, uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int cap256, uint32_t big_thr) {
   extern __shared__ uint32_t lds[];
   __shared__ uint32_t last;
   const int tid = threadIdx.x;
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
 
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   dispatch_block(topk_idx, (int64_t)T * k, E, nbits, k, lds, counts, offsets, perm, inv_perm, src_of,
-                 work, mtiles, big_thr);
+                 work, mtiles, cap256, big_thr);
 }
 
 bool router_fused_applies(int64_t T, int E, int k) {
@@ -78,8 +78,8 @@ hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const floa
                                int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx,
                                uint16_t *topk_w, uint32_t *counters, uint32_t *counts,
                                uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
-                               uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int big_thr,
-                               hipStream_t st) {
+                               uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int cap256,
+                               int big_thr, hipStream_t st) {
   int nbits = 0;
   while ((1 << nbits) < E) ++nbits;
   dim3 grid((unsigned)T, (unsigned)((E + kDispWaves - 1) / kDispWaves));
@@ -87,7 +87,7 @@ hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const floa
 #define MI_FUSED(NV)                                                                              \
   router_fused_kernel<NV><<<grid, kDispThreads, lds, st>>>(                                        \
       x, wg, bias, (int)T, H, E, k, mode, logits, topk_idx, topk_w, counters, nbits, counts,      \
-      offsets, perm, inv_perm, src_of, work, mtiles, (uint32_t)big_thr)
+      offsets, perm, inv_perm, src_of, work, mtiles, cap256, (uint32_t)big_thr)
   if (E <= 64) MI_FUSED(1);
   else if (E <= 128) MI_FUSED(2);
   else if (E <= 256) MI_FUSED(4);

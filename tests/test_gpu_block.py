@@ -93,3 +93,11 @@ def test_fused_router_equals_the_separate_kernels(orc):
                                 (dbg["inv_perm"], inv, "inv_perm")):
             assert torch.equal(got.reshape(want.shape), want), f"{name} at T={T}"
         assert torch.equal(dbg["topk_w"].view(torch.int16), sc.view(torch.int16)), f"scores at T={T}"
+
+
+@pytest.mark.parametrize("T,E,k,bits,zipf", [(192, 8, 2, 4, None), (200, 8, 2, 4, 0.8), (700, 8, 2, 8, None),
+                                             (333, 16, 4, 4, 1.2), (1100, 4, 1, 4, None)])
+def test_tile_classes(orc, T, E, k, bits, zipf):
+    # segments of 9 rows and more are cut into 256-, 128- and 64-row tiles, shorter ones stream:
+    # these shapes put segments into every class, with remainders on both sides of each boundary
+    _run_case(orc, 256, E, k, 384, bits, T, 0, seed=31 + T, zipf_s=zipf)

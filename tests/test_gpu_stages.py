@@ -159,11 +159,11 @@ def test_errors_reach_the_caller(m):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("M", [1, 5, 47, 48, 300])
+@pytest.mark.parametrize("M", [1, 5, 8, 9, 64, 65, 130, 300])
 def test_quantized_matmul_equals_matmul_on_dequantized(orc, bits, M):
     """The identity of the reference's test_quantized_matmul (mlx-rs/src/ops/quantization.rs:318-342),
     in the transposed layout QuantizedLinear uses: qmm(x, w_q, s, b) == x @ dequantize(w_q, s, b)^T.
-    Rows below 48 run on the streaming kernel, from 48 on on the tiled one."""
+    Up to 8 rows run on the streaming kernel, more on the tiled one (64-, 128- and 256-row tiles)."""
     import mlx_rs_amd as m
     rng = np.random.default_rng(50 + M)
     N, K = 192, 256

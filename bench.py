@@ -23,9 +23,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # HBM bytes per launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE scaled by
-# what the same counters read for a plain copy kernel (profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt);
+# what the same counters read for a plain copy kernel (profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt,
+# profiles/qmm_large_kernel_prefill_tokens4096_counters.txt);
 # counters cannot be read from inside this script, so the figure is carried here per workload.
-MEASURED_TRAFFIC_BYTES = {"decode": 2.060e8}
+MEASURED_TRAFFIC_BYTES = {"decode": 2.057e8, "prefill": 5.10e8}
 
 
 def parse():

@@ -106,6 +106,22 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
                    void *workspace, size_t workspace_bytes, const mi_moe_debug_out *dbg,
                    void *stream);
 
+/* The block between its neighbours in a decoder layer (mlx-lm/src/models/qwen3.rs:310-325:
+ * r = post_attention_layernorm(h); r = mlp(r); out = h + r): out = x + moe(rms_norm(x, norm_weight,
+ * eps)), with the residual add folded into the combine (one rounding) and the normalised rows
+ * kept in the workspace.  norm_weight: bf16 [H].  out must not alias x.  Same workspace as
+ * mi_moe_forward.  Replaces mlx_fast_rms_norm (mlx-rs/src/fast.rs:190-207) and mlx_add around
+ * the block. */
+int mi_moe_forward_residual(mi_moe_handle h, const uint16_t *x, const uint16_t *norm_weight,
+                            float eps, int64_t T, uint16_t *out, void *workspace,
+                            size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream);
+
+/* RMS normalisation over the last axis on its own: out = weight * x * rsqrt(mean(x^2) + eps)
+ * (mlx_fast_rms_norm, mlx-rs/src/fast.rs:190-207; nn::RmsNorm, nn/normalization.rs:233-275).
+ * x, out: bf16 [T, hidden]; weight: bf16 [hidden]. */
+int mi_moe_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T,
+                    int32_t hidden, uint16_t *out, void *stream);
+
 /* The same forward with a HIP event recorded on `stream` before the first launch and
  * after each stage; waits for the last one and returns the MI_MOE_N_STAGES elapsed times
  * in milliseconds (host array): router logits, router select, dispatch, gate/up + SwiGLU,

@@ -14,7 +14,8 @@ STAGE_NAMES = ("router_logits", "router_select", "dispatch", "gate_up_swiglu", "
 # every symbol include/mi_moe.h declares
 EXPORTS = (
     "mi_moe_last_error", "mi_moe_set_error_handler", "mi_moe_version", "mi_moe_create",
-    "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_forward_timed",
+    "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_forward_residual",
+    "mi_moe_rms_norm", "mi_moe_forward_timed",
     "mi_moe_route_workspace_size",
     "mi_moe_route", "mi_moe_dispatch_workspace_size", "mi_moe_dispatch",
     "mi_moe_gather_qmm_workspace_size", "mi_moe_gather_qmm",
@@ -84,6 +85,8 @@ def load_library():
         "mi_moe_workspace_size": [C.POINTER(Config), i64, C.POINTER(sz)],
         "mi_moe_forward": [vp, vp, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
         "mi_moe_forward_timed": [vp, vp, i64, vp, vp, sz, vp, C.POINTER(C.c_float)],
+        "mi_moe_forward_residual": [vp, vp, vp, C.c_float, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
+        "mi_moe_rms_norm": [vp, vp, C.c_float, i64, i32, vp, vp],
         "mi_moe_route_workspace_size": [i32, i64, C.POINTER(sz)],
         "mi_moe_route": [vp, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp, vp, sz, vp],
         "mi_moe_dispatch_workspace_size": [i32, i64, C.POINTER(sz)],

@@ -88,7 +88,7 @@ struct ForwardWs {
   int max_mtiles;
   bool tiled;
   void *disp_scratch;
-  uint16_t *hh, *y, *xperm;
+  uint16_t *hh, *y, *xperm, *xnorm;
   size_t bytes;
 };
 
@@ -117,6 +117,7 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.hh = cv.take<uint16_t>((size_t)P * c.intermediate);
   f.y = cv.take<uint16_t>((size_t)P * c.hidden);
   f.xperm = cv.take<uint16_t>(f.tiled && c.bits == 4 ? (size_t)T * c.hidden : 0);
+  f.xnorm = cv.take<uint16_t>((size_t)T * c.hidden);  // rms_norm(x) of the residual variant
   f.bytes = cv.off;
   return f;
 }
@@ -185,9 +186,10 @@ int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *
 
 // The launch sequence of one forward.  ev: nullptr, or kStages + 1 events recorded on the
 // stream before the first launch and after each stage.
-static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
+static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16_t *out, void *workspace,
                         size_t workspace_bytes, const mi_moe_debug_out *dbg, hipStream_t st,
-                        hipEvent_t *ev) {
+                        hipEvent_t *ev, const uint16_t *norm_weight = nullptr, float eps = 0.f) {
+  const uint16_t *x = x_in;
   if (!h) return fail("forward: handle is NULL");
   if (T < 0) return fail("forward: negative token count");
   if (T == 0) return 0;
@@ -207,6 +209,10 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
     if (ev) MI_HIP(hipEventRecord(ev[++stage], st));     \
   } while (0)
   if (ev) MI_HIP(hipEventRecord(ev[0], st));
+  if (norm_weight) {  // the block's input is rms_norm(x); x itself is added back in the combine
+    MI_HIP(launch_rms_norm(x_in, norm_weight, eps, T, c.hidden, f.xnorm, st));
+    x = f.xnorm;
+  }
 
   if (router_fused_applies(T, c.n_experts, c.top_k)) {
     // decode: one launch for the three stages (the stage times then all land in the first)
@@ -271,7 +277,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
   a.K = c.intermediate;
   MI_HIP(launch_grouped_qmm(a, false, st));
   MI_STAGE_DONE();
-  MI_HIP(launch_combine(f.y, f.topk_w, nullptr, T, c.top_k, c.hidden, out, st));
+  MI_HIP(launch_combine(f.y, f.topk_w, nullptr, T, c.top_k, c.hidden, norm_weight ? x_in : nullptr, out, st));
   MI_STAGE_DONE();
 #undef MI_STAGE_DONE
 
@@ -289,6 +295,28 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t 
 int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
                    size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream) {
   return forward_impl(h, x, T, out, workspace, workspace_bytes, dbg, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int mi_moe_forward_residual(mi_moe_handle h, const uint16_t *x, const uint16_t *norm_weight, float eps,
+                            int64_t T, uint16_t *out, void *workspace, size_t workspace_bytes,
+                            const mi_moe_debug_out *dbg, void *stream) {
+  if (!norm_weight || !aligned16(norm_weight)) return fail("forward_residual: norm_weight must be non-NULL and 16-byte aligned");
+  if (!(eps >= 0.f)) return fail("forward_residual: eps must be non-negative");
+  if (x == out) return fail("forward_residual: out must not alias x (x is read again at the end)");
+  return forward_impl(h, x, T, out, workspace, workspace_bytes, dbg, static_cast<hipStream_t>(stream), nullptr,
+                      norm_weight, eps);
+}
+
+int mi_moe_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int32_t hidden,
+                    uint16_t *out, void *stream) {
+  if (T < 0) return fail("rms_norm: negative row count");
+  if (hidden <= 0 || hidden % 8) return fail("rms_norm: hidden must be a positive multiple of 8, got %d", hidden);
+  if (!(eps >= 0.f)) return fail("rms_norm: eps must be non-negative");
+  if (T == 0) return 0;
+  if (!x || !weight || !out) return fail("rms_norm: x, weight and out must be non-NULL");
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(out)) return fail("rms_norm: pointers must be 16-byte aligned");
+  MI_HIP(launch_rms_norm(x, weight, eps, T, hidden, out, static_cast<hipStream_t>(stream)));
+  return 0;
 }
 
 int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
@@ -511,7 +539,7 @@ int mi_moe_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *in
   if (T == 0) return 0;
   if (!y || !scores || !out) return fail("combine: y, scores and out must be non-NULL");
   if (!aligned16(y) || !aligned16(out)) return fail("combine: y and out must be 16-byte aligned");
-  MI_HIP(launch_combine(y, scores, inv_perm, T, top_k, hidden, out, static_cast<hipStream_t>(stream)));
+  MI_HIP(launch_combine(y, scores, inv_perm, T, top_k, hidden, nullptr, out, static_cast<hipStream_t>(stream)));
   return 0;
 }
 

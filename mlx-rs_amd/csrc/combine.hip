@@ -10,7 +10,8 @@ namespace mi_moe {
 
 __global__ __launch_bounds__(256) void combine_kernel(
     const uint16_t *__restrict__ y, const uint16_t *__restrict__ scores,
-    const uint32_t *__restrict__ inv_perm, int64_t T, int k, int H, uint16_t *__restrict__ out) {
+    const uint32_t *__restrict__ inv_perm, int64_t T, int k, int H,
+    const uint16_t *__restrict__ residual, uint16_t *__restrict__ out) {
   const int64_t t = blockIdx.x;
   const int h = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (h >= H) return;
@@ -26,6 +27,15 @@ __global__ __launch_bounds__(256) void combine_kernel(
       acc[2 * i + 1] += sc * bf16hi_to_f32(u[i]);
     }
   }
+  if (residual) {  // h + mlp(...): the block's neighbour in a decoder layer, added before the one rounding
+    const uint4 v = *reinterpret_cast<const uint4 *>(residual + t * H + h);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      acc[2 * i] = bf16lo_to_f32(u[i]) + acc[2 * i];
+      acc[2 * i + 1] = bf16hi_to_f32(u[i]) + acc[2 * i + 1];
+    }
+  }
   uint4 o;
   o.x = pack_bf16x2(acc[0], acc[1]);
   o.y = pack_bf16x2(acc[2], acc[3]);
@@ -35,10 +45,58 @@ __global__ __launch_bounds__(256) void combine_kernel(
 }
 
 hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
-                          int64_t T, int k, int H, uint16_t *out, hipStream_t st) {
+                          int64_t T, int k, int H, const uint16_t *residual, uint16_t *out,
+                          hipStream_t st) {
   if (T == 0) return hipSuccess;
   dim3 grid((unsigned)T, (unsigned)((H / 8 + 255) / 256));
-  combine_kernel<<<grid, 256, 0, st>>>(y, scores, inv_perm, T, k, H, out);
+  combine_kernel<<<grid, 256, 0, st>>>(y, scores, inv_perm, T, k, H, residual, out);
+  return hipGetLastError();
+}
+
+// RMS normalisation over the last axis (mlx_fast_rms_norm, mlx-rs/src/fast.rs:190-207;
+// nn::RmsNorm, mlx-rs/src/nn/normalization.rs:233-275): one wave per row.  The mean of squares is
+// accumulated in double over exact products (any order gives the same float), 1 / sqrt in
+// correctly rounded float operations, one rounding to bf16: the bits of the host-side checker,
+// which the selection of experts downstream depends on.
+__global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t *__restrict__ x,
+                                                       const uint16_t *__restrict__ weight, float eps,
+                                                       int64_t T, int H, uint16_t *__restrict__ out) {
+  const int lane = lane_id();
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const uint16_t *xr = x + t * H;
+  double ss = 0.0;
+  for (int h = lane * 8; h < H; h += kWave * 8) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(xr + h);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const double a = (double)bf16lo_to_f32(u[i]), b = (double)bf16hi_to_f32(u[i]);
+      ss = __builtin_fma(a, a, ss);
+      ss = __builtin_fma(b, b, ss);
+    }
+  }
+  ss = wave_sum_f64(ss);
+  const float mean = (float)(ss / (double)H);
+  const float rstd = 1.0f / sqrtf(mean + eps);
+  for (int h = lane * 8; h < H; h += kWave * 8) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(xr + h);
+    const uint4 w = *reinterpret_cast<const uint4 *>(weight + h);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w}, wu[4] = {w.x, w.y, w.z, w.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = bf16lo_to_f32(u[i]) * rstd, hi = bf16hi_to_f32(u[i]) * rstd;
+      o[i] = pack_bf16x2(bf16lo_to_f32(wu[i]) * lo, bf16hi_to_f32(wu[i]) * hi);
+    }
+    *reinterpret_cast<uint4 *>(out + t * H + h) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
+hipError_t launch_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int H,
+                           uint16_t *out, hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  rms_norm_kernel<<<(unsigned)((T + 3) / 4), 256, 0, st>>>(x, weight, eps, T, H, out);
   return hipGetLastError();
 }
 

@@ -169,7 +169,10 @@ hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t
 hipError_t launch_swiglu(const uint16_t *g, const uint16_t *u, int64_t n, uint16_t *out,
                          hipStream_t st);
 hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
-                          int64_t T, int k, int H, uint16_t *out, hipStream_t st);
+                          int64_t T, int k, int H, const uint16_t *residual, uint16_t *out,
+                          hipStream_t st);
+hipError_t launch_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int H,
+                           uint16_t *out, hipStream_t st);
 hipError_t launch_quantize(const float *w, int64_t rows, int64_t cols, int group, int bits,
                            uint32_t *q, uint16_t *s, uint16_t *b, hipStream_t st);
 hipError_t launch_dequantize(const uint32_t *q, const uint16_t *s, const uint16_t *b,

@@ -279,6 +279,25 @@ inline Result<Array> gather_qmm(const Array &x, const Array &w, const Array &sca
 
 }  // namespace ops
 
+namespace fast {
+
+// rms_norm(x, weight, eps): weight * x * rsqrt(mean(x^2) + eps) over the last axis
+// (mlx-rs/src/fast.rs:190-207).  x: bf16 [..., H]; weight: bf16 [H].
+inline Result<Array> rms_norm(const Array &x, const Array &weight, float eps, Stream s = {}) {
+  if (auto e = detail::want(x, Dtype::Bfloat16, "rms_norm", "x")) return *e;
+  if (auto e = detail::want(weight, Dtype::Bfloat16, "rms_norm", "weight")) return *e;
+  if (x.ndim() < 1 || weight.size() != x.dim(-1)) return Exception("rms_norm: weight must match the last axis of x");
+  auto out = Array::empty(x.shape(), Dtype::Bfloat16);
+  if (out.is_err()) return out;
+  const int64_t H = x.dim(-1);
+  if (mi_moe_rms_norm(x.ptr<uint16_t>(), weight.ptr<uint16_t>(), eps, x.size() / H, (int32_t)H,
+                      out.value().ptr<uint16_t>(), s.as_ptr()))
+    return detail::last_error("rms_norm");
+  return out;
+}
+
+}  // namespace fast
+
 namespace nn {
 
 // E quantized matrices with a leading expert axis: the fields of QuantizedLinear
@@ -348,6 +367,24 @@ class SparseMoeBlock {
     if (mi_moe_forward(handle_, x.ptr<uint16_t>(), T, out.value().ptr<uint16_t>(),
                        workspace_.data(), workspace_.nbytes(), dbg, s.as_ptr()))
       return detail::last_error("forward");
+    return out;
+  }
+
+  // x + forward(rms_norm(x, norm_weight, eps)): the block between its neighbours in a decoder layer
+  // (mlx-lm/src/models/qwen3.rs:310-325), one call
+  Result<Array> forward_residual(const Array &x, const Array &norm_weight, float eps, Stream s = {}) {
+    if (auto e = detail::want(x, Dtype::Bfloat16, "forward_residual", "x")) return *e;
+    if (auto e = detail::want(norm_weight, Dtype::Bfloat16, "forward_residual", "norm_weight")) return *e;
+    if (x.ndim() < 1 || x.dim(-1) != cfg_.hidden || norm_weight.size() != cfg_.hidden)
+      return Exception("forward_residual: last dimension must be " + std::to_string(cfg_.hidden));
+    const int64_t T = x.size() / cfg_.hidden;
+    if (auto r = reserve(T > 0 ? T : 1); r.is_err()) return r.error();
+    auto out = Array::empty(x.shape(), Dtype::Bfloat16);
+    if (out.is_err()) return out;
+    if (mi_moe_forward_residual(handle_, x.ptr<uint16_t>(), norm_weight.ptr<uint16_t>(), eps, T,
+                                out.value().ptr<uint16_t>(), workspace_.data(), workspace_.nbytes(), nullptr,
+                                s.as_ptr()))
+      return detail::last_error("forward_residual");
     return out;
   }
 

@@ -85,7 +85,12 @@ class SparseMoeBlock:
             self._ws_tokens = tokens
         return self._ws
 
-    def forward(self, x, debug=False, out=None):
+    def forward_residual(self, x, norm_weight, eps=1e-5, debug=False, out=None):
+        """x + self(rms_norm(x, norm_weight, eps)): the block with the layer norm in front of it and
+        the residual add behind it (mlx-lm/src/models/qwen3.rs:310-325) in one call."""
+        return self.forward(x, debug=debug, out=out, _norm=(_need(norm_weight, torch.bfloat16, "norm_weight"), eps))
+
+    def forward(self, x, debug=False, out=None, _norm=None):
         """x: bf16 [..., H] -> bf16 [..., H].  With debug=True also returns the routing
         arrays (topk_idx, topk_w, counts, offsets, perm, inv_perm)."""
         _need(x, torch.bfloat16, "x")
@@ -108,8 +113,15 @@ class SparseMoeBlock:
                        inv_perm=torch.empty(P, dtype=torch.int32, device=dev))
             dbg_struct = capi.DebugOut(*[dbg[n].data_ptr() for n in
                                          ("topk_idx", "topk_w", "counts", "offsets", "perm", "inv_perm")])
-        check(self._lib.mi_moe_forward(self._handle, _ptr(x2), T, _ptr(out), _ptr(ws), ws.numel(),
-                                       None if dbg_struct is None else C.byref(dbg_struct), _stream()))
+        dbg_arg = None if dbg_struct is None else C.byref(dbg_struct)
+        if _norm is None:
+            check(self._lib.mi_moe_forward(self._handle, _ptr(x2), T, _ptr(out), _ptr(ws), ws.numel(), dbg_arg,
+                                           _stream()))
+        else:
+            if _norm[0].numel() != c.hidden:
+                raise capi.MoeError(f"forward_residual: norm_weight must have {c.hidden} elements")
+            check(self._lib.mi_moe_forward_residual(self._handle, _ptr(x2), _ptr(_norm[0]), float(_norm[1]), T,
+                                                    _ptr(out), _ptr(ws), ws.numel(), dbg_arg, _stream()))
         out = out.reshape(x.shape)
         return (out, dbg) if debug else out
 

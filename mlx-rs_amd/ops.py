@@ -114,6 +114,21 @@ def quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4
     return y.reshape(*x.shape[:-1], N)
 
 
+def rms_norm(x, weight, eps=1e-5):
+    """fast::rms_norm (mlx-rs/src/fast.rs:190-207): weight * x * rsqrt(mean(x^2) + eps) over the last
+    axis.  x: bf16 [..., H]; weight: bf16 [H]."""
+    lib = load_library()
+    _need(x, torch.bfloat16, "x")
+    _need(weight, torch.bfloat16, "weight")
+    H = x.shape[-1]
+    if weight.numel() != H:
+        raise capi.MoeError(f"rms_norm: weight must have {H} elements, got {weight.numel()}")
+    x2 = x.reshape(-1, H)
+    out = torch.empty_like(x2)
+    check(lib.mi_moe_rms_norm(_ptr(x2), _ptr(weight), float(eps), x2.shape[0], H, _ptr(out), _stream()))
+    return out.reshape(x.shape)
+
+
 def route(x, router_w, top_k, score_mode=capi.SCORE_SOFTMAX_THEN_TOPK_RENORM, router_bias=None,
           return_logits=False):
     """Gate Linear + softmax(precise) + top-k + scores in one call (what an mlx-lm MoE block

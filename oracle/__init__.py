@@ -227,13 +227,22 @@ def combine(y, sc, inv_perm, strict=False):
     return out
 
 
+def rms_norm(x, weight, eps=1e-5):
+    x, weight = _c(x, np.uint16), _c(weight, np.uint16)
+    T, H = x.shape
+    out = np.empty((T, H), np.uint16)
+    lib().orc_rms_norm(_p(x), _p(weight), C.c_float(eps), C.c_int64(T), H, _p(out))
+    return out
+
+
 def make_config(hidden, n_experts, top_k, intermediate, bits=4, group_size=64, score_mode=0):
     return Config(hidden, n_experts, top_k, intermediate, bits, group_size, score_mode)
 
 
-def moe_forward(cfg, weights, x, strict=False, n_threads=8, debug=True):
+def moe_forward(cfg, weights, x, strict=False, n_threads=8, debug=True, norm_weight=None, eps=1e-5):
     """weights: dict with router_w (uint16 [E,H]), router_bias (float32 [E] or None) and
     gate/up/down each a (w uint32, scales uint16, biases uint16) tuple.
+    With norm_weight (uint16 [H]) the result is x + moe(rms_norm(x, norm_weight, eps)).
     Returns (out uint16 [T,H], dict of routing arrays)."""
     x = _c(x, np.uint16)
     T = x.shape[0]
@@ -255,6 +264,12 @@ def moe_forward(cfg, weights, x, strict=False, n_threads=8, debug=True):
              counts=np.empty(cfg.n_experts, np.uint32), offsets=np.empty(cfg.n_experts + 1, np.uint32),
              perm=np.empty(P, np.uint32), inv_perm=np.empty(P, np.uint32))
     dbg = DebugOut(*[_p(d[n]) for n in ("topk_idx", "topk_w", "counts", "offsets", "perm", "inv_perm")])
-    _chk(lib().orc_moe_forward(C.byref(cfg), C.byref(W), _p(x), C.c_int64(T), _p(out),
-                               C.byref(dbg) if debug else None, int(strict), int(n_threads)))
+    if norm_weight is None:
+        _chk(lib().orc_moe_forward(C.byref(cfg), C.byref(W), _p(x), C.c_int64(T), _p(out),
+                                   C.byref(dbg) if debug else None, int(strict), int(n_threads)))
+    else:
+        nw = _c(norm_weight, np.uint16)
+        _chk(lib().orc_moe_forward_residual(C.byref(cfg), C.byref(W), _p(x), _p(nw), C.c_float(eps),
+                                            C.c_int64(T), _p(out), C.byref(dbg) if debug else None,
+                                            int(strict), int(n_threads)))
     return out, d

@@ -414,8 +414,9 @@ void orc_swiglu_f32(const float *gate, const float *up, int64_t n, uint16_t *out
 /* ------------------------------------------------------------------ R8 combine
  * (y * scores[..., None]).sum(-2): slots added in order s = 0..k-1 in fp32
  * (ops/arithmetic.rs:138-160, ops/reduction.rs:260-276). */
-void orc_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
-                 int64_t T, int k, int H, int strict, uint16_t *out) {
+static void combine_impl(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
+                         int64_t T, int k, int H, int strict, const uint16_t *residual,
+                         uint16_t *out) {
 #pragma omp parallel for schedule(static)
   for (int64_t t = 0; t < T; ++t)
     for (int h = 0; h < H; ++h) {
@@ -426,17 +427,26 @@ void orc_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_
         if (strict) v = orc_bf16_to_f32(orc_f32_to_bf16(v));
         acc += v;
       }
+      if (residual) {  /* h + mlp(...): one more bf16 op in the op-by-op sequence */
+        if (strict) acc = orc_bf16_to_f32(orc_f32_to_bf16(acc));
+        acc = orc_bf16_to_f32(residual[t * H + h]) + acc;
+      }
       out[t * H + h] = orc_f32_to_bf16(acc);
     }
+}
+
+void orc_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
+                 int64_t T, int k, int H, int strict, uint16_t *out) {
+  combine_impl(y, scores, inv_perm, T, k, H, strict, NULL, out);
 }
 
 /* ------------------------------------------------------------------ M: the block
  * mlx-lm's sparse MoE block (SwitchGLU over gather_qmm): route, sort pairs by expert,
  * gate/up products, SwiGLU, down product, unsort, weighted sum over slots.  The block
  * sits where the dense Mlp sits in mlx-lm/src/models/qwen3.rs:204-255,321-324. */
-int orc_moe_forward(const orc_config *cfg, const orc_weights *w, const uint16_t *x,
-                    int64_t T, uint16_t *out, const orc_debug_out *dbg, int strict,
-                    int n_threads) {
+static int moe_forward_impl(const orc_config *cfg, const orc_weights *w, const uint16_t *x,
+                            int64_t T, uint16_t *out, const orc_debug_out *dbg, int strict,
+                            int n_threads, const uint16_t *residual) {
   const int H = cfg->hidden, E = cfg->n_experts, k = cfg->top_k, I = cfg->intermediate;
   const int bits = cfg->bits, group = cfg->group_size;
   if (!(bits == 4 || bits == 8)) return fail("forward: bits must be 4 or 8");
@@ -509,7 +519,7 @@ int orc_moe_forward(const orc_config *cfg, const orc_weights *w, const uint16_t 
     free(rg);
     free(xf);
   }
-  orc_combine(y, scores, inv, T, k, H, strict, out);
+  combine_impl(y, scores, inv, T, k, H, strict, residual, out);
 
   if (dbg) {
     if (dbg->topk_idx) memcpy(dbg->topk_idx, inds, sizeof(uint32_t) * (size_t)P);
@@ -526,3 +536,48 @@ done:
   free(y);
   return rc;
 }
+
+int orc_moe_forward(const orc_config *cfg, const orc_weights *w, const uint16_t *x,
+                    int64_t T, uint16_t *out, const orc_debug_out *dbg, int strict,
+                    int n_threads) {
+  return moe_forward_impl(cfg, w, x, T, out, dbg, strict, n_threads, NULL);
+}
+
+/* RMS normalisation over the last axis: y = weight * x * rsqrt(mean(x^2) + eps)
+ * (mlx-rs/src/nn/normalization.rs:233-275 -> fast::rms_norm, mlx-rs/src/fast.rs:190-207).
+ * The mean of squares is accumulated in double (exact products, so the value does not depend on
+ * the summation order), rounded to float; 1/sqrt in correctly rounded float operations; one
+ * rounding to bf16 at the end. */
+void orc_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int H,
+                  uint16_t *out) {
+  for (int64_t t = 0; t < T; ++t) {
+    const uint16_t *xr = x + t * H;
+    double ss = 0.0;
+    for (int h = 0; h < H; ++h) {
+      const double v = (double)orc_bf16_to_f32(xr[h]);
+      ss += v * v;
+    }
+    const float mean = (float)(ss / (double)H);
+    const float rstd = 1.0f / sqrtf(mean + eps);
+    for (int h = 0; h < H; ++h) {
+      const float xn = orc_bf16_to_f32(xr[h]) * rstd;
+      out[t * H + h] = orc_f32_to_bf16(orc_bf16_to_f32(weight[h]) * xn);
+    }
+  }
+}
+
+/* The block between its neighbours in a decoder layer (mlx-lm/src/models/qwen3.rs:310-325):
+ * out = x + moe(rms_norm(x, norm_weight, eps)).  strict: the block's result is rounded to bf16
+ * before the add (two arrays in MLX); otherwise the add happens in the combine's accumulator. */
+int orc_moe_forward_residual(const orc_config *cfg, const orc_weights *w, const uint16_t *x,
+                             const uint16_t *norm_weight, float eps, int64_t T, uint16_t *out,
+                             const orc_debug_out *dbg, int strict, int n_threads) {
+  const int H = cfg->hidden;
+  uint16_t *xn = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)(T * H + 1));
+  if (!xn) return fail("forward_residual: out of memory");
+  orc_rms_norm(x, norm_weight, eps, T, H, xn);
+  int rc = moe_forward_impl(cfg, w, xn, T, out, dbg, strict, n_threads, x);
+  free(xn);
+  return rc;
+}
+

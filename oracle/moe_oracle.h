@@ -42,6 +42,11 @@
  *   orc_swiglu                     pinned: closed form, sigmoid KATs
  *                                  ops/arithmetic.rs:2577-2600.
  *   orc_combine                    pinned: closed form, slot-permutation invariance.
+ *   orc_rms_norm                   pinned: closed form in float64 numpy, torch (float32 compute), the
+ *                                  statistic of the reference test fast.rs:304-324 (uniform(0,1)
+ *                                  input, unit weight: mean 0.8729 +- 0.0175).  Where MLX rounds
+ *                                  inside its kernel (once at the end here) is "parity unpinned".
+ *   orc_moe_forward_residual       pinned: composition of orc_rms_norm, orc_moe_forward and an add.
  *   orc_moe_forward                pinned: composition of the above vs an independent
  *                                  fp64 numpy restatement of the whole block.  No test
  *                                  in the reference exercises an MoE composition
@@ -151,6 +156,15 @@ void orc_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_
 int orc_moe_forward(const orc_config *cfg, const orc_weights *w, const uint16_t *x,
                     int64_t T, uint16_t *out, const orc_debug_out *dbg, int strict,
                     int n_threads);
+
+/* next to the path: RMS normalisation (mlx-rs/src/nn/normalization.rs:233-275, fast.rs:190-207) and
+ * the block between its neighbours in a decoder layer, out = x + moe(rms_norm(x))
+ * (mlx-lm/src/models/qwen3.rs:310-325). */
+void orc_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int H,
+                  uint16_t *out);
+int orc_moe_forward_residual(const orc_config *cfg, const orc_weights *w, const uint16_t *x,
+                             const uint16_t *norm_weight, float eps, int64_t T, uint16_t *out,
+                             const orc_debug_out *dbg, int strict, int n_threads);
 
 const char *orc_last_error(void);
 

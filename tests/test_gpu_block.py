@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import (assert_close_bf16, bits_u16, bits_u32, bf16_tensor, device_block, errors,
+from helpers import (assert_close_bf16, bits_u16, bits_u32, bf16_tensor, device_block, errors, f32_of_bits,
                      host_layer, host_tokens)
 
 pytestmark = pytest.mark.gpu
@@ -101,3 +101,37 @@ def test_tile_classes(orc, T, E, k, bits, zipf):
     # segments of 9 rows and more are cut into 256-, 128- and 64-row tiles, shorter ones stream:
     # these shapes put segments into every class, with remainders on both sides of each boundary
     _run_case(orc, 256, E, k, 384, bits, T, 0, seed=31 + T, zipf_s=zipf)
+
+
+@pytest.mark.parametrize("T,H,E,k,I,bits,mode,zipf", [(1, 256, 8, 2, 512, 4, 0, None), (32, 2048, 128, 8, 768, 4, 0, None),
+                                                      (300, 256, 16, 4, 256, 8, 2, 1.0)])
+def test_norm_and_residual_around_the_block(orc, T, H, E, k, I, bits, mode, zipf):
+    """mi_moe_forward_residual: x + moe(rms_norm(x)).  The normalised rows carry the selection, so
+    routing must still match the oracle bit for bit; rms_norm on its own is bit-exact too."""
+    import mlx_rs_amd as m
+    print(f"residual case T={T} H={H} E={E} k={k} I={I} bits={bits} mode={mode}", flush=True)
+    W = host_layer(orc, H, E, k, I, bits, seed=40 + T, zipf_s=zipf)
+    x = host_tokens(orc, T, H, seed=40 + T)
+    nw = orc.f32_to_bf16(np.random.default_rng(T).normal(1.0, 0.2, H).astype(np.float32))
+    blk = device_block(m, m.MoeConfig(H, E, k, I, bits, 64, mode), W)
+    xd, nwd = bf16_tensor(x, "cuda"), bf16_tensor(nw, "cuda")
+    out, dbg = blk.forward_residual(xd, nwd, 1e-6, debug=True)
+    xn = m.ops.rms_norm(xd, nwd, 1e-6)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_u16(xn), orc.rms_norm(x, nw, 1e-6)), "rms_norm differs from the oracle"
+    ocfg = orc.make_config(H, E, k, I, bits, 64, mode)
+    ref_s, d = orc.moe_forward(ocfg, W, x, strict=True, n_threads=16, norm_weight=nw, eps=1e-6)
+    ref_f, _ = orc.moe_forward(ocfg, W, x, strict=False, n_threads=16, norm_weight=nw, eps=1e-6)
+    for name in ("topk_idx", "counts", "perm"):
+        assert np.array_equal(bits_u32(dbg[name]).reshape(d[name].shape), d[name]), name
+    assert np.array_equal(bits_u16(dbg["topk_w"]), d["topk_w"])
+    scale = max(1.0, float(np.abs(f32_of_bits(ref_s)).max()) / 4)  # |x| reaches 4: one bf16 ulp there is 3e-2
+    assert_close_bf16(bits_u16(out), ref_f, max_abs=2e-2 * scale, what="vs oracle (fused rounding points)")
+    assert_close_bf16(bits_u16(out), ref_s, max_abs=2e-2 * scale, what="vs oracle (op-by-op rounding)")
+    # and it is the plain forward on rms_norm(x) plus x, up to the one rounding that is saved
+    y = blk.forward(xn)
+    torch.cuda.synchronize()
+    want = (xd.float() + y.float()).bfloat16()
+    assert (out.float() - want.float()).abs().max().item() <= 2e-2 * scale
+    with pytest.raises(m.MoeError, match="alias"):
+        blk.forward_residual(xd, nwd, 1e-6, out=xd)

@@ -209,14 +209,16 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     if (ev) MI_HIP(hipEventRecord(ev[++stage], st));     \
   } while (0)
   if (ev) MI_HIP(hipEventRecord(ev[0], st));
+  const bool fused_router = router_fused_applies(T, c.n_experts, c.top_k);
   if (norm_weight) {  // the block's input is rms_norm(x); x itself is added back in the combine
-    MI_HIP(launch_rms_norm(x_in, norm_weight, eps, T, c.hidden, f.xnorm, st));
-    x = f.xnorm;
+    if (!fused_router) MI_HIP(launch_rms_norm(x_in, norm_weight, eps, T, c.hidden, f.xnorm, st));
+    x = f.xnorm;      // decode: written by the router kernel below
   }
 
-  if (router_fused_applies(T, c.n_experts, c.top_k)) {
+  if (fused_router) {
     // decode: one launch for the three stages (the stage times then all land in the first)
-    MI_HIP(launch_router_fused(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, c.top_k,
+    MI_HIP(launch_router_fused(x_in, h->w.router_w, h->w.router_bias, norm_weight, eps, f.xnorm, T, c.hidden,
+                               c.n_experts, c.top_k,
                                c.score_mode, f.logits, f.topk_idx, f.topk_w, h->counters, f.counts, f.offsets,
                                f.perm, f.inv_perm, f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles,
                                kTileMinRows, st));

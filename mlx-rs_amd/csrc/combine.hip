@@ -4,7 +4,7 @@
 // (mlx-rs/src/ops/indexing/mod.rs:386-401, ops/shapes.rs:398-415,466-484,
 // ops/arithmetic.rs:138-160, ops/reduction.rs:260-276): every output element is one
 // thread's fp32 sum over the k slots in slot order: no atomics, run-to-run identical.
-#include "common.hpp"
+#include "router_dev.hpp"
 
 namespace mi_moe {
 
@@ -61,36 +61,13 @@ hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint3
 __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t *__restrict__ x,
                                                        const uint16_t *__restrict__ weight, float eps,
                                                        int64_t T, int H, uint16_t *__restrict__ out) {
-  const int lane = lane_id();
   const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
   const uint16_t *xr = x + t * H;
-  double ss = 0.0;
-  for (int h = lane * 8; h < H; h += kWave * 8) {
-    const uint4 v = *reinterpret_cast<const uint4 *>(xr + h);
-    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const double a = (double)bf16lo_to_f32(u[i]), b = (double)bf16hi_to_f32(u[i]);
-      ss = __builtin_fma(a, a, ss);
-      ss = __builtin_fma(b, b, ss);
-    }
-  }
-  ss = wave_sum_f64(ss);
-  const float mean = (float)(ss / (double)H);
-  const float rstd = 1.0f / sqrtf(mean + eps);
-  for (int h = lane * 8; h < H; h += kWave * 8) {
-    const uint4 v = *reinterpret_cast<const uint4 *>(xr + h);
-    const uint4 w = *reinterpret_cast<const uint4 *>(weight + h);
-    const uint32_t u[4] = {v.x, v.y, v.z, v.w}, wu[4] = {w.x, w.y, w.z, w.w};
-    uint32_t o[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float lo = bf16lo_to_f32(u[i]) * rstd, hi = bf16hi_to_f32(u[i]) * rstd;
-      o[i] = pack_bf16x2(bf16lo_to_f32(wu[i]) * lo, bf16hi_to_f32(wu[i]) * hi);
-    }
-    *reinterpret_cast<uint4 *>(out + t * H + h) = make_uint4(o[0], o[1], o[2], o[3]);
-  }
+  const float rstd = row_rstd_wave(xr, H, eps);
+  for (int h = lane_id() * 8; h < H; h += kWave * 8)
+    *reinterpret_cast<uint4 *>(out + t * H + h) =
+        rms_norm8(*reinterpret_cast<const uint4 *>(xr + h), *reinterpret_cast<const uint4 *>(weight + h), rstd);
 }
 
 hipError_t launch_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int H,

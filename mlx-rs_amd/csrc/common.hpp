@@ -70,21 +70,52 @@ __device__ __forceinline__ float det_expf(float x) {
 // ---------------------------------------------------------------- wave helpers
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
-__device__ __forceinline__ double shfl_xor_f64(double v, int m) {
-  int lo = __double2loint(v), hi = __double2hiint(v);
-  lo = __shfl_xor(lo, m, kWave);
-  hi = __shfl_xor(hi, m, kWave);
+// Wave-wide reductions whose result every lane holds.  Inside a row of 16 lanes the partners come
+// through DPP (quad permutes, then the half-row and row mirrors: a few cycles each, no LDS traffic);
+// the four row results are read as scalars and combined in the same fixed order by every lane.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, CTRL, 0xf, 0xf, true);
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+  const int lo = __builtin_amdgcn_mov_dpp(__double2loint(v), CTRL, 0xf, 0xf, true);
+  const int hi = __builtin_amdgcn_mov_dpp(__double2hiint(v), CTRL, 0xf, 0xf, true);
   return __hiloint2double(hi, lo);
 }
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+
+__device__ __forceinline__ double readlane_f64(double v, int l) {
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), l),
+                          __builtin_amdgcn_readlane(__double2loint(v), l));
+}
 __device__ __forceinline__ double wave_sum_f64(double v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_f64(v, m);
-  return v;
+  v += dpp_f64<kDppXor1>(v);
+  v += dpp_f64<kDppXor2>(v);
+  v += dpp_f64<kDppHalfMirror>(v);
+  v += dpp_f64<kDppMirror>(v);
+  return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
 }
 __device__ __forceinline__ float wave_max_f32(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
-  return v;
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppXor1>(__float_as_uint(v))));
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppXor2>(__float_as_uint(v))));
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppHalfMirror>(__float_as_uint(v))));
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppMirror>(__float_as_uint(v))));
+  const uint32_t u = __float_as_uint(v);
+  const float a = __uint_as_float(__builtin_amdgcn_readlane(u, 0)), b = __uint_as_float(__builtin_amdgcn_readlane(u, 16));
+  const float c = __uint_as_float(__builtin_amdgcn_readlane(u, 32)), d = __uint_as_float(__builtin_amdgcn_readlane(u, 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  uint32_t o;
+  o = dpp_u32<kDppXor1>(v); v = o > v ? o : v;
+  o = dpp_u32<kDppXor2>(v); v = o > v ? o : v;
+  o = dpp_u32<kDppHalfMirror>(v); v = o > v ? o : v;
+  o = dpp_u32<kDppMirror>(v); v = o > v ? o : v;
+  const uint32_t a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+  const uint32_t c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+  const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+  return ab > cd ? ab : cd;
 }
 
 // ---------------------------------------------------------------- M-tile lists
@@ -150,9 +181,11 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
                            uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int cap256, int big_thr,
                            void *scratch, hipStream_t st);
 // decode-sized batches: logits + selection + dispatch in one launch.  counters: 1 +
-// kFusedRouterMaxTokens zero-initialised words that the kernel leaves zeroed again.
+// kFusedRouterMaxTokens zero-initialised words that the kernel leaves zeroed again.  norm_w != nullptr:
+// the rows are RMS-normalised first (weight norm_w, eps) and kept in xnorm.
 bool router_fused_applies(int64_t T, int E, int k);
-hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const float *bias, int64_t T,
+hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const float *bias,
+                               const uint16_t *norm_w, float eps, uint16_t *xnorm, int64_t T,
                                int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx,
                                uint16_t *topk_w, uint32_t *counters, uint32_t *counts,
                                uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,

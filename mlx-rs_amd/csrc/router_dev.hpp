@@ -24,6 +24,56 @@ __device__ __forceinline__ double logit_wave(const uint16_t *__restrict__ xr,
   return wave_sum_f64(acc);
 }
 
+// 1 / sqrt(mean(x^2) + eps) of a row, by one wave: the mean of squares in fp64 over exact products,
+// the rest in correctly rounded float operations (the bits of the host-side checker).
+__device__ __forceinline__ float row_rstd_wave(const uint16_t *__restrict__ xr, int H, float eps) {
+  double ss = 0.0;
+  for (int h = lane_id() * 8; h < H; h += kWave * 8) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(xr + h);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const double a = (double)bf16lo_to_f32(u[i]), b = (double)bf16hi_to_f32(u[i]);
+      ss = __builtin_fma(a, a, ss);
+      ss = __builtin_fma(b, b, ss);
+    }
+  }
+  ss = wave_sum_f64(ss);
+  return 1.0f / sqrtf((float)(ss / (double)H) + eps);
+}
+// eight normalised values of a row: bf16(weight * (x * rstd)), packed
+__device__ __forceinline__ uint4 rms_norm8(uint4 v, uint4 w, float rstd) {
+  const uint32_t u[4] = {v.x, v.y, v.z, v.w}, wu[4] = {w.x, w.y, w.z, w.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float lo = bf16lo_to_f32(u[i]) * rstd, hi = bf16hi_to_f32(u[i]) * rstd;
+    o[i] = pack_bf16x2(bf16lo_to_f32(wu[i]) * lo, bf16hi_to_f32(wu[i]) * hi);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+// logit of (rms_norm(token row), expert row); the wave optionally writes the normalised row
+__device__ __forceinline__ double logit_wave_norm(const uint16_t *__restrict__ xr,
+                                                  const uint16_t *__restrict__ wr,
+                                                  const uint16_t *__restrict__ norm_w, float eps, int H,
+                                                  uint16_t *xn_out) {
+  const float rstd = row_rstd_wave(xr, H, eps);
+  double acc = 0.0;
+  for (int h = lane_id() * 8; h < H; h += kWave * 8) {
+    const uint4 xv = rms_norm8(*reinterpret_cast<const uint4 *>(xr + h),
+                               *reinterpret_cast<const uint4 *>(norm_w + h), rstd);
+    if (xn_out) *reinterpret_cast<uint4 *>(xn_out + h) = xv;
+    const uint4 wv = *reinterpret_cast<const uint4 *>(wr + h);
+    const uint32_t xu[4] = {xv.x, xv.y, xv.z, xv.w}, wu[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      acc = __builtin_fma((double)bf16lo_to_f32(xu[q]), (double)bf16lo_to_f32(wu[q]), acc);
+      acc = __builtin_fma((double)bf16hi_to_f32(xu[q]), (double)bf16hi_to_f32(wu[q]), acc);
+    }
+  }
+  return wave_sum_f64(acc);
+}
+
 // float -> unsigned key whose unsigned order is the float order; -0 is mapped to +0 so
 // that the two zeros tie (and the lower expert id wins) as they do in a float compare.
 __device__ __forceinline__ uint32_t ordered_key(float f) {
@@ -35,15 +85,6 @@ __device__ __forceinline__ float key_to_float(uint32_t k) {
   uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
   return __uint_as_float(u);
 }
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) {
-    const uint32_t o = __shfl_xor(v, m, kWave);
-    v = o > v ? o : v;
-  }
-  return v;
-}
-
 // Softmax, top-k and scores of one token by one wave.  Lane l holds experts l, l+64, ... (NV of
 // them).  COHERENT: the logits were written by other workgroups of the same launch.
 // The values the selection compares are exact in bf16 (rounded probabilities, or the logits

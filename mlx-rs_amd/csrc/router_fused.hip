@@ -23,6 +23,7 @@ namespace mi_moe {
 template <int NV>
 __global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg, const float *__restrict__ bias,
+    const uint16_t *__restrict__ norm_w, float eps, uint16_t *__restrict__ xnorm,
     int T, int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx, uint16_t *topk_w,
     uint32_t *counters, int nbits, uint32_t *counts, uint32_t *offsets, uint32_t *perm,
     uint32_t *inv_perm, uint32_t *src_of, uint32_t *work, uint32_t *mtiles, int cap256, uint32_t big_thr) {
@@ -34,7 +35,11 @@ __global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
   const int e = blockIdx.y * kDispWaves + wave;
 
   if (e < E) {
-    double s = logit_wave(x + (int64_t)t * H, wg + (int64_t)e * H, H);
+    // with a norm weight the token row is normalised first; every wave derives the same
+    // normalised values, one of them (first workgroup of the token, first wave) keeps the row
+    double s = norm_w ? logit_wave_norm(x + (int64_t)t * H, wg + (int64_t)e * H, norm_w, eps, H,
+                                        blockIdx.y == 0 && wave == 0 ? xnorm + (int64_t)t * H : nullptr)
+                      : logit_wave(x + (int64_t)t * H, wg + (int64_t)e * H, H);
     if (lane_id() == 0) {
       if (bias) s += (double)bias[e];
       store_agent(logits + (int64_t)t * E + e, f32_to_bf16((float)s));
@@ -74,7 +79,8 @@ bool router_fused_applies(int64_t T, int E, int k) {
   return T >= 1 && T <= kFusedRouterMaxTokens && T * k <= kSingleMaxP;
 }
 
-hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const float *bias, int64_t T,
+hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const float *bias,
+                               const uint16_t *norm_w, float eps, uint16_t *xnorm, int64_t T,
                                int H, int E, int k, int mode, uint16_t *logits, uint32_t *topk_idx,
                                uint16_t *topk_w, uint32_t *counters, uint32_t *counts,
                                uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm,
@@ -86,7 +92,7 @@ hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const floa
   const size_t lds = (size_t)(3 + kDispWaves) * E * sizeof(uint32_t);
 #define MI_FUSED(NV)                                                                              \
   router_fused_kernel<NV><<<grid, kDispThreads, lds, st>>>(                                        \
-      x, wg, bias, (int)T, H, E, k, mode, logits, topk_idx, topk_w, counters, nbits, counts,      \
+      x, wg, bias, norm_w, eps, xnorm, (int)T, H, E, k, mode, logits, topk_idx, topk_w, counters, nbits, counts,      \
       offsets, perm, inv_perm, src_of, work, mtiles, cap256, (uint32_t)big_thr)
   if (E <= 64) MI_FUSED(1);
   else if (E <= 128) MI_FUSED(2);

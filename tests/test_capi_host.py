@@ -87,6 +87,21 @@ def test_null_and_range_checks(lib):
     assert lib.mi_moe_quantize(None, 2, 100, 64, 4, None, None, None, None) != 0
     assert "divisible" in m.capi.last_error()
     assert lib.mi_moe_dequantize(None, None, None, 2, 128, 64, 3, None, None) != 0
+    # entry points next to the path
+    n2 = C.c_size_t(7)
+    assert lib.mi_moe_quantized_matmul_workspace_size(-1, 128, 4, C.byref(n2)) != 0 and n2.value == 7
+    assert lib.mi_moe_quantized_matmul_workspace_size(300, 256, 4, C.byref(n2)) == 0 and n2.value > 300 * 256 * 2
+    assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 64, 128, 0, 64, 4, None, None, 0, None) != 0
+    assert "transpose" in m.capi.last_error()
+    assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 60, 128, 1, 64, 4, None, None, 0, None) != 0
+    assert "N must" in m.capi.last_error()
+    assert lib.mi_moe_quantized_matmul(None, None, None, None, 0, 64, 128, 1, 64, 4, None, None, 0, None) == 0
+    assert lib.mi_moe_rms_norm(None, None, 1e-5, 4, 100, None, None) != 0 and "hidden" in m.capi.last_error()
+    assert lib.mi_moe_rms_norm(None, None, -1.0, 4, 128, None, None) != 0 and "eps" in m.capi.last_error()
+    assert lib.mi_moe_rms_norm(None, None, 1e-5, 4, 128, None, None) != 0
+    assert lib.mi_moe_rms_norm(None, None, 1e-5, 0, 128, None, None) == 0
+    assert lib.mi_moe_forward_residual(None, None, None, 1e-5, 1, None, None, 0, None, None) != 0
+    assert "norm_weight" in m.capi.last_error()
     # empty inputs succeed without touching memory
     assert lib.mi_moe_swiglu(None, None, 0, None, None) == 0
     assert lib.mi_moe_combine(None, None, None, 0, 2, 64, None, None) == 0

@@ -135,3 +135,58 @@ def test_norm_and_residual_around_the_block(orc, T, H, E, k, I, bits, mode, zipf
     assert (out.float() - want.float()).abs().max().item() <= 2e-2 * scale
     with pytest.raises(m.MoeError, match="alias"):
         blk.forward_residual(xd, nwd, 1e-6, out=xd)
+
+
+@pytest.mark.parametrize("T", [4, 300])
+def test_graph_replays_equal_eager(orc, T):
+    """A forward captured into a HIP graph (decode: the one-launch router with its self-resetting
+    arrival counters; prefill: the tiled kernels) gives the eager result on every replay, with
+    eager forwards of other sizes and synchronisations in between."""
+    import mlx_rs_amd as m
+    H, E, k, I = 256, 16, 4, 256
+    W = host_layer(orc, H, E, k, I, 4, seed=77)
+    blk = device_block(m, m.MoeConfig(H, E, k, I), W)
+    x = bf16_tensor(host_tokens(orc, T, H, seed=77), "cuda")
+    other = bf16_tensor(host_tokens(orc, 7, H, seed=78), "cuda")
+    blk.reserve(max(T, 7))
+    eager = blk.forward(x).clone()
+    out = torch.empty_like(x)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        blk.forward(x, out=out)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        blk.forward(x, out=out)
+    for rep in range(4):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {rep} differs from the eager result"
+        blk.forward(other)  # eager work through the same handle and workspace between the replays
+        torch.cuda.synchronize()
+
+
+def test_two_handles_on_two_streams(orc):
+    """Handles are independent: two layers running concurrently on two streams (each with its own
+    workspace) give what they give one after the other."""
+    import mlx_rs_amd as m
+    H, E, k, I, T = 256, 16, 4, 256, 16
+    blks, xs, refs = [], [], []
+    for i in range(2):
+        W = host_layer(orc, H, E, k, I, 4, seed=90 + i)
+        blks.append(device_block(m, m.MoeConfig(H, E, k, I), W))
+        xs.append(bf16_tensor(host_tokens(orc, T, H, seed=90 + i), "cuda"))
+        refs.append(blks[i].forward(xs[i]).clone())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.empty_like(xs[0]), torch.empty_like(xs[1])]
+    for rep in range(20):
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                blks[i].forward(xs[i], out=outs[i])
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert torch.equal(outs[i].view(torch.int16), refs[i].view(torch.int16)), f"handle {i}"

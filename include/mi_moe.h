@@ -154,7 +154,9 @@ int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts
  * for j < n_idx: y[j] (M x N) = x[lhs[j]] (M x K) . dequantize(w[rhs[j]])^T.
  * x: bf16 [x_batch, M, K]; w: [E, N, K*bits/32]; y: bf16 [n_idx, M, N].
  * lhs_indices NULL = identity (j), as an absent mlx_array; rhs_indices required.
- * transpose must be non-zero (the layout every mlx-lm switch layer uses);
+ * transpose non-zero is the layout every mlx-lm switch layer uses and the tuned path; with
+ * transpose = 0, w is [E, K, N*bits/32] with scales, biases [E, K, N/group_size] (K x N matrices
+ * quantised along N, N a multiple of 64), served by a plain kernel that needs no workspace.
  * sorted_indices is a hint, results do not depend on it.
  * workspace >= mi_moe_gather_qmm_workspace_size. */
 int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M, size_t *bytes);
@@ -169,7 +171,9 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
  * QuantizedLinear::forward calls it with transpose = true, mlx-rs/src/nn/quantized.rs:363-386):
  * y (M x N) = x (M x K) . dequantize(w)^T on the same kernels as gather_qmm (one matrix, every row).
  * x: bf16 [M, K]; w: [N, K*bits/32]; scales, biases: bf16 [N, K/group_size]; y: bf16 [M, N].
- * transpose must be non-zero.  workspace >= mi_moe_quantized_matmul_workspace_size. */
+ * transpose = 0 (the op's own default; test_quantized_matmul, ops/quantization.rs:318-342):
+ * w [K, N*bits/32], scales, biases [K, N/group_size], y = x . dequantize(w), a plain kernel.
+ * workspace >= mi_moe_quantized_matmul_workspace_size (transpose = 0 needs none). */
 int mi_moe_quantized_matmul_workspace_size(int64_t M, int32_t K, int32_t bits, size_t *bytes);
 int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
                             const uint16_t *biases, int64_t M, int32_t N, int32_t K,

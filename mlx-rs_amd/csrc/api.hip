@@ -416,9 +416,21 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
                       uint16_t *y, void *workspace, size_t workspace_bytes, void *stream) {
   (void)sorted_indices;  // a hint in MLX; the segments are rebuilt here either way
   (void)x_batch;
-  if (!transpose) return fail("gather_qmm: transpose = false is not supported (weights must be [E, N, K*bits/32])");
   if (bits != 4 && bits != 8) return fail("gather_qmm: bits must be 4 or 8, got %d", bits);
   if (group_size != 64) return fail("gather_qmm: group_size must be 64, got %d", group_size);
+  if (!transpose) {  // w [E, K, N*bits/32]: the plain kernel, no workspace
+    if (K <= 0) return fail("gather_qmm: K must be positive, got %d", K);
+    if (N <= 0 || N % 64) return fail("gather_qmm: with transpose = false N must be a positive multiple of 64, got %d", N);
+    if (M < 1) return fail("gather_qmm: M must be positive, got %d", M);
+    if (n_experts < 1) return fail("gather_qmm: n_experts must be positive, got %d", n_experts);
+    if (n_idx < 0 || n_idx * M > (int64_t)1 << 30) return fail("gather_qmm: index count out of range");
+    if (n_idx == 0) return 0;
+    if (!x || !w || !scales || !biases || !y) return fail("gather_qmm: x, w, scales, biases and y must be non-NULL");
+    if (!rhs_indices) return fail("gather_qmm: rhs_indices is required");
+    MI_HIP(launch_qmm_nt(x, w, scales, biases, lhs_indices, rhs_indices, n_idx * M, M, N, K, group_size, bits, y,
+                         static_cast<hipStream_t>(stream)));
+    return 0;
+  }
   if (K <= 0 || K % 64) return fail("gather_qmm: K must be a positive multiple of 64, got %d", K);
   if (bits == 4 && K % 128) return fail("gather_qmm: 4-bit weights need K to be a multiple of 128, got %d", K);
   if (N <= 0 || N % 16) return fail("gather_qmm: N must be a positive multiple of 16, got %d", N);
@@ -483,9 +495,18 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
                             const uint16_t *biases, int64_t M, int32_t N, int32_t K, int32_t transpose,
                             int32_t group_size, int32_t bits, uint16_t *y, void *workspace,
                             size_t workspace_bytes, void *stream) {
-  if (!transpose) return fail("quantized_matmul: transpose = false is not supported (weights must be [N, K*bits/32])");
   if (bits != 4 && bits != 8) return fail("quantized_matmul: bits must be 4 or 8, got %d", bits);
   if (group_size != 64) return fail("quantized_matmul: group_size must be 64, got %d", group_size);
+  if (!transpose) {  // w [K, N*bits/32]: the plain kernel, no workspace
+    if (K <= 0) return fail("quantized_matmul: K must be positive, got %d", K);
+    if (N <= 0 || N % 64) return fail("quantized_matmul: with transpose = false N must be a positive multiple of 64, got %d", N);
+    if (M < 0 || M > (int64_t)1 << 30) return fail("quantized_matmul: row count out of range");
+    if (M == 0) return 0;
+    if (!x || !w || !scales || !biases || !y) return fail("quantized_matmul: x, w, scales, biases and y must be non-NULL");
+    MI_HIP(launch_qmm_nt(x, w, scales, biases, nullptr, nullptr, M, 1, N, K, group_size, bits, y,
+                         static_cast<hipStream_t>(stream)));
+    return 0;
+  }
   if (K <= 0 || K % 64) return fail("quantized_matmul: K must be a positive multiple of 64, got %d", K);
   if (bits == 4 && K % 128) return fail("quantized_matmul: 4-bit weights need K to be a multiple of 128, got %d", K);
   if (N <= 0 || N % 16) return fail("quantized_matmul: N must be a positive multiple of 16, got %d", N);

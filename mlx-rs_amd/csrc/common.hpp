@@ -206,6 +206,9 @@ hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint3
                           hipStream_t st);
 hipError_t launch_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int H,
                            uint16_t *out, hipStream_t st);
+hipError_t launch_qmm_nt(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                         const uint16_t *biases, const uint32_t *lhs, const uint32_t *rhs, int64_t rows,
+                         int M, int N, int K, int group, int bits, uint16_t *y, hipStream_t st);
 hipError_t launch_quantize(const float *w, int64_t rows, int64_t cols, int group, int bits,
                            uint32_t *q, uint16_t *s, uint16_t *b, hipStream_t st);
 hipError_t launch_dequantize(const uint32_t *q, const uint16_t *s, const uint16_t *b,

@@ -94,4 +94,62 @@ hipError_t launch_dequantize(const uint32_t *q, const uint16_t *s, const uint16_
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Quantized product with an UNTRANSPOSED weight (transpose = false, the default of
+// ops::quantized_matmul, mlx-rs/src/ops/quantization.rs:91-122, and the layout of the reference's
+// test_quantized_matmul, :318-342): w holds K x N matrices quantised along N,
+//   w [E, K, N*bits/32], scales / biases [E, K, N/group];  y[r] (N) = x[src(r)] (K) . W_hat[e(r)].
+// Not a layout any mlx-lm switch layer uses: a plain, correct kernel (one thread per packed word
+// of an output row, fp32 accumulation in k order), not a tuned one.
+template <int BITS>
+__global__ __launch_bounds__(256) void qmm_nt_kernel(const uint16_t *__restrict__ x,
+                                                     const uint32_t *__restrict__ w,
+                                                     const uint16_t *__restrict__ scales,
+                                                     const uint16_t *__restrict__ biases,
+                                                     const uint32_t *__restrict__ lhs,
+                                                     const uint32_t *__restrict__ rhs, int M, int N, int K,
+                                                     int group, uint16_t *__restrict__ y) {
+  constexpr int CPW = 32 / BITS;  // codes per word
+  const int64_t r = blockIdx.x;   // output row = j * M + m
+  const int wi = blockIdx.y * 256 + threadIdx.x;
+  const int wpr = N / CPW;
+  if (wi >= wpr) return;
+  const int64_t j = r / M;
+  const int m = (int)(r % M);
+  const int64_t e = rhs ? (int64_t)rhs[j] : 0;
+  const int64_t xb = lhs ? (int64_t)lhs[j] : j;
+  const uint16_t *xr = x + (xb * M + m) * K;
+  const int gpr = N / group, g = wi * CPW / group;
+  const uint32_t *wp = w + e * K * wpr + wi;
+  const uint16_t *sp = scales + e * K * gpr + g, *bp = biases + e * K * gpr + g;
+  float acc[CPW];
+#pragma unroll
+  for (int c = 0; c < CPW; ++c) acc[c] = 0.f;
+  for (int k = 0; k < K; ++k) {
+    const uint32_t word = wp[(int64_t)k * wpr];
+    const float sc = bf16_to_f32(sp[(int64_t)k * gpr]), bi = bf16_to_f32(bp[(int64_t)k * gpr]);
+    const float xv = bf16_to_f32(xr[k]);
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const float qv = (float)((word >> (c * BITS)) & ((1u << BITS) - 1u));
+      acc[c] = __builtin_fmaf(xv, __builtin_fmaf(sc, qv, bi), acc[c]);
+    }
+  }
+  uint16_t *yo = y + r * N + (int64_t)wi * CPW;
+#pragma unroll
+  for (int c = 0; c < CPW; c += 2)
+    *reinterpret_cast<uint32_t *>(yo + c) = pack_bf16x2(acc[c], acc[c + 1]);
+}
+
+hipError_t launch_qmm_nt(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                         const uint16_t *biases, const uint32_t *lhs, const uint32_t *rhs, int64_t rows,
+                         int M, int N, int K, int group, int bits, uint16_t *y, hipStream_t st) {
+  if (rows == 0) return hipSuccess;
+  const int wpr = N * bits / 32;
+  dim3 grid((unsigned)rows, (unsigned)((wpr + 255) / 256));
+  if (bits == 4) qmm_nt_kernel<4><<<grid, 256, 0, st>>>(x, w, scales, biases, lhs, rhs, M, N, K, group, y);
+  else qmm_nt_kernel<8><<<grid, 256, 0, st>>>(x, w, scales, biases, lhs, rhs, M, N, K, group, y);
+  return hipGetLastError();
+}
+
 }  // namespace mi_moe

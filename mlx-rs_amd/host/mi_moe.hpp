@@ -207,8 +207,9 @@ inline Result<Array> dequantize(const Array &w, const Array &scales, const Array
 }
 
 // quantized_matmul(x, w, scales, biases, transpose, group_size, bits): x bf16 [M, K]; w u32
-// [N, K*bits/32]; returns bf16 [M, N].  The reference's default is transpose = false; only the
-// transposed layout (the one QuantizedLinear uses) is implemented, so it is the default here.
+// [N, K*bits/32] (transpose = false: [K, N*bits/32]); returns bf16 [M, N].  The reference's default is
+// transpose = false; the transposed layout (the one QuantizedLinear uses) is the tuned one and the
+// default here.
 inline Result<Array> quantized_matmul(const Array &x, const Array &w, const Array &scales,
                                       const Array *biases = nullptr, std::optional<bool> transpose = {},
                                       std::optional<int32_t> group_size = {},
@@ -221,7 +222,7 @@ inline Result<Array> quantized_matmul(const Array &x, const Array &w, const Arra
   if (!biases) return Exception("quantized_matmul: biases are required in affine mode");
   if (x.ndim() != 2 || w.ndim() != 2) return Exception("quantized_matmul: x must be [M, K] and w [N, K*bits/32]");
   const int64_t M = x.dim(0);
-  const int32_t K = (int32_t)x.dim(1), N = (int32_t)w.dim(0);
+  const int32_t K = (int32_t)x.dim(1), N = tr ? (int32_t)w.dim(0) : (int32_t)(w.dim(1) * 32 / b);
   size_t ws_bytes = 0;
   if (mi_moe_quantized_matmul_workspace_size(M, K, b, &ws_bytes)) return detail::last_error("quantized_matmul");
   auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);
@@ -258,7 +259,7 @@ inline Result<Array> gather_qmm(const Array &x, const Array &w, const Array &sca
     return Exception("gather_qmm: x must be [batch, M, K] and w [E, N, K*bits/32]");
   const int64_t n_idx = rhs_indices->size(), xb = x.dim(0);
   const int32_t M = (int32_t)x.dim(1), K = (int32_t)x.dim(2);
-  const int32_t E = (int32_t)w.dim(0), N = (int32_t)w.dim(1);
+  const int32_t E = (int32_t)w.dim(0), N = tr ? (int32_t)w.dim(1) : (int32_t)(w.dim(2) * 32 / b);
   size_t ws_bytes = 0;
   if (mi_moe_gather_qmm_workspace_size(E, n_idx, M, &ws_bytes)) return detail::last_error("gather_qmm");
   auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);

@@ -73,7 +73,7 @@ def gather_qmm(x, w, scales, biases, lhs_indices=None, rhs_indices=None, transpo
     if x.dim() != 3 or w.dim() != 3:
         raise capi.MoeError("gather_qmm: x must be [batch, M, K] and w [E, N, K*bits/32]")
     xb, M, K = x.shape
-    E, N = w.shape[0], w.shape[1]
+    E, N = w.shape[0], (w.shape[1] if transpose else w.shape[2] * 32 // bits)
     if rhs_indices is None:
         raise capi.MoeError("gather_qmm: rhs_indices is required")
     n_idx = rhs_indices.numel()
@@ -92,15 +92,16 @@ def gather_qmm(x, w, scales, biases, lhs_indices=None, rhs_indices=None, transpo
 
 def quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4):
     """ops::quantized_matmul (mlx-rs/src/ops/quantization.rs:91-122) the way QuantizedLinear calls
-    it (transpose = true, mlx-rs/src/nn/quantized.rs:363-386; the op's own default is false, which
-    this build does not implement).  x: bf16 [..., K]; w: int32 [N, K*bits/32]; returns bf16 [..., N]."""
+    it (transpose = true, mlx-rs/src/nn/quantized.rs:363-386): x: bf16 [..., K]; w: int32
+    [N, K*bits/32]; returns bf16 [..., N].  transpose = False (the op's own default): w int32
+    [K, N*bits/32], scales/biases [K, N/group_size], a plain kernel."""
     lib = load_library()
     _need(x, torch.bfloat16, "x")
     _need(w, torch.int32, "w")
     if w.dim() != 2 or x.dim() < 1:
         raise capi.MoeError("quantized_matmul: x must be [..., K] and w [N, K*bits/32]")
     K = x.shape[-1]
-    N = w.shape[0]
+    N = w.shape[0] if transpose else w.shape[1] * 32 // bits
     x2 = x.reshape(-1, K)
     M = x2.shape[0]
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)

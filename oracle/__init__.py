@@ -185,12 +185,24 @@ def dispatch(flat, E):
     return counts, offsets, perm, inv
 
 
-def gather_qmm(x, w, s, b, lhs, rhs, bits=4, group=64, n_threads=8, want="f32"):
-    """x: uint16 [x_batch, M, K]; w: uint32 [E, N, K*bits/32]; returns [n_idx, M, N]."""
+def gather_qmm(x, w, s, b, lhs, rhs, bits=4, group=64, n_threads=8, want="f32", transpose=True):
+    """x: uint16 [x_batch, M, K]; w: uint32 [E, N, K*bits/32] (transpose=False: [E, K, N*bits/32]);
+    returns [n_idx, M, N]."""
     x, w = _c(x, np.uint16), _c(w, np.uint32)
     s, b = _c(s, np.uint16), _c(b, np.uint16)
     xb, M, K = x.shape
     E, N = w.shape[0], w.shape[1]
+    if not transpose:
+        N = w.shape[2] * 32 // bits
+        rhs = np.ascontiguousarray(np.asarray(rhs).reshape(-1).astype(np.uint32))
+        if lhs is not None:
+            lhs = np.ascontiguousarray(np.asarray(lhs).reshape(-1).astype(np.uint32))
+        n_idx = rhs.size
+        yf = np.empty((n_idx, M, N), np.float32) if want == "f32" else None
+        yb = np.empty((n_idx, M, N), np.uint16) if want == "bf16" else None
+        _chk(lib().orc_gather_qmm_nt(_p(x), _p(w), _p(s), _p(b), _p(lhs), _p(rhs), C.c_int64(n_idx),
+                                     C.c_int64(xb), M, N, K, E, bits, group, _p(yf), _p(yb)))
+        return yf if want == "f32" else yb
     rhs = np.ascontiguousarray(np.asarray(rhs).reshape(-1).astype(np.uint32))
     if lhs is not None:
         lhs = np.ascontiguousarray(np.asarray(lhs).reshape(-1).astype(np.uint32))

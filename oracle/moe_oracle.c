@@ -394,6 +394,45 @@ int orc_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
   return 0;
 }
 
+/* transpose = false (the default of ops::quantized_matmul, ops/quantization.rs:91-122; the layout of
+ * the reference's test_quantized_matmul, :318-342): w holds a K x N matrix quantised along N,
+ * w: [E, K, N*bits/32], scales/biases: [E, K, N/group]; out[j] (M x N) = x[lhs[j]] (M x K) . W_hat[rhs[j]].
+ * fp32 accumulation in k order. */
+int orc_gather_qmm_nt(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                      const uint16_t *biases, const uint32_t *lhs, const uint32_t *rhs,
+                      int64_t n_idx, int64_t x_batch, int M, int N, int K, int E, int bits,
+                      int group, float *y_f32, uint16_t *y_bf16) {
+  if (!(bits == 4 || bits == 8 || bits == 2)) return fail("gather_qmm: bits must be 2, 4 or 8");
+  if (group <= 0 || N % group != 0) return fail("gather_qmm: N must be divisible by group_size");
+  for (int64_t j = 0; j < n_idx; ++j) {
+    if (rhs[j] >= (uint32_t)E) return fail("gather_qmm: rhs index out of range");
+    if ((lhs ? (int64_t)lhs[j] : j) >= x_batch) return fail("gather_qmm: lhs index out of range");
+  }
+  const int64_t wpr = (int64_t)N * bits / 32, gpr = N / group;
+  float *wrow = (float *)malloc(sizeof(float) * (size_t)N);
+  float *acc = (float *)malloc(sizeof(float) * (size_t)M * N);
+  if (!wrow || !acc) return fail("gather_qmm: out of memory");
+  for (int64_t j = 0; j < n_idx; ++j) {
+    const int64_t xb = lhs ? lhs[j] : j, e = rhs[j];
+    for (int64_t i = 0; i < (int64_t)M * N; ++i) acc[i] = 0.0f;
+    for (int k = 0; k < K; ++k) {
+      dequant_row(w + (e * K + k) * wpr, scales + (e * K + k) * gpr, biases + (e * K + k) * gpr, N,
+                  bits, group, wrow);
+      for (int m = 0; m < M; ++m) {
+        const float xv = orc_bf16_to_f32(x[(xb * M + m) * K + k]);
+        for (int n = 0; n < N; ++n) acc[(int64_t)m * N + n] += xv * wrow[n];
+      }
+    }
+    for (int64_t i = 0; i < (int64_t)M * N; ++i) {
+      if (y_f32) y_f32[j * M * N + i] = acc[i];
+      if (y_bf16) y_bf16[j * M * N + i] = orc_f32_to_bf16(acc[i]);
+    }
+  }
+  free(wrow);
+  free(acc);
+  return 0;
+}
+
 /* ------------------------------------------------------------------ R7 SwiGLU
  * nn::silu = compile(x * sigmoid(x)) (nn/activation.rs:142-144,876-880), then
  * multiply by `up`.  Op by op on bf16 arrays every result is a bf16 value. */

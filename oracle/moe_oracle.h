@@ -39,6 +39,10 @@
  *   orc_gather_qmm                 pinned: identity of ops/quantization.rs:345-423
  *                                  (== gather_mm on dequantised weights), fp64 numpy,
  *                                  E=1 -> torch matmul, unit-scale integer case (exact).
+ *   orc_gather_qmm_nt              pinned: the identity of ops/quantization.rs:318-342
+ *                                  (== x @ dequantize(w)) in fp64 numpy, and agreement with
+ *                                  orc_gather_qmm on the transposed, re-quantised-free case K = N
+ *                                  groups aligned (unit scales).
  *   orc_swiglu                     pinned: closed form, sigmoid KATs
  *                                  ops/arithmetic.rs:2577-2600.
  *   orc_combine                    pinned: closed form, slot-permutation invariance.
@@ -142,6 +146,11 @@ int orc_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
                    const uint16_t *biases, const uint32_t *lhs, const uint32_t *rhs,
                    int64_t n_idx, int64_t x_batch, int M, int N, int K, int E, int bits,
                    int group, float *y_f32, uint16_t *y_bf16, int n_threads);
+/* the same with transpose = false: w [E, K, N*bits/32] holds K x N matrices quantised along N */
+int orc_gather_qmm_nt(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                      const uint16_t *biases, const uint32_t *lhs, const uint32_t *rhs,
+                      int64_t n_idx, int64_t x_batch, int M, int N, int K, int E, int bits,
+                      int group, float *y_f32, uint16_t *y_bf16);
 /* R7 silu(gate) * up.  strict != 0: bf16 round after every MLX op
  * (nn/activation.rs:142-144,876-880), else one round at the end. */
 void orc_swiglu_bf16(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out);

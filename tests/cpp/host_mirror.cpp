@@ -133,8 +133,8 @@ static int run_forward(const std::string &dir) {
   dump(dir + "/gq.bin", g);
   // library-side refusal surfaces as an error value with its text
   auto bad2 = ops::gather_qmm(x.reshape({T, 1, H}), gate.weight, gate.scales, &gate.biases, &lhs, &rhs,
-                              false, 64, (int32_t)bits, false);
-  EXPECT(bad2.is_err() && contains(bad2.error(), "transpose"));
+                              true, 32, (int32_t)bits, false);
+  EXPECT(bad2.is_err() && contains(bad2.error(), "group_size"));
 
   // ops::quantize / ops::dequantize with the defaults (group 64, 4 bits)
   Array wf = load(dir, "wf.bin", {qrows, qcols}, Dtype::Float32);

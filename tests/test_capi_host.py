@@ -76,9 +76,9 @@ def test_null_and_range_checks(lib):
     assert lib.mi_moe_route(None, None, None, 4, 250, 8, 2, 0, None, None, None, None, 0, None) != 0
     assert "hidden" in m.capi.last_error()
     assert lib.mi_moe_dispatch(None, 8, 4, None, None, None, None, None, 0, None) != 0
-    assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 64, 64, 3, 0, 64, 4, 0,
+    assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 96, 64, 3, 0, 64, 4, 0,
                                  None, None, 0, None) != 0
-    assert "transpose" in m.capi.last_error()
+    assert "transpose" in m.capi.last_error()      # untransposed weights need N to be a multiple of 64
     assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 64, 64, 3, 1, 64, 5, 0,
                                  None, None, 0, None) != 0
     assert "bits" in m.capi.last_error()
@@ -91,7 +91,7 @@ def test_null_and_range_checks(lib):
     n2 = C.c_size_t(7)
     assert lib.mi_moe_quantized_matmul_workspace_size(-1, 128, 4, C.byref(n2)) != 0 and n2.value == 7
     assert lib.mi_moe_quantized_matmul_workspace_size(300, 256, 4, C.byref(n2)) == 0 and n2.value > 300 * 256 * 2
-    assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 64, 128, 0, 64, 4, None, None, 0, None) != 0
+    assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 96, 128, 0, 64, 4, None, None, 0, None) != 0
     assert "transpose" in m.capi.last_error()
     assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 60, 128, 1, 64, 4, None, None, 0, None) != 0
     assert "N must" in m.capi.last_error()

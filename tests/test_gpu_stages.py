@@ -184,6 +184,40 @@ def test_quantized_matmul_equals_matmul_on_dequantized(orc, bits, M):
     yo = orc.gather_qmm(x.reshape(M, 1, K), q[None], s[None], b[None], None, np.zeros(M, np.uint32),
                         bits=bits, want="f32").reshape(M, N)
     assert np.abs(yo - ref).max() <= 1e-4
-    with pytest.raises(m.MoeError, match="transpose"):
-        m.ops.quantized_matmul(bf16_tensor(x, "cuda"), i32_tensor(q, "cuda"), bf16_tensor(s, "cuda"),
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_untransposed_quantized_matmul_and_gather_qmm(orc, bits):
+    """transpose = false, the layout of the reference's test_quantized_matmul
+    (mlx-rs/src/ops/quantization.rs:318-342: m 32, n 128, k 128, group 64, w = normal * 1/sqrt(k),
+    quantised along n): qmm(x, w_q, s, b, false) == x @ dequantize(w_q, s, b).  The reference's bound
+    is 1e-3 on float32 inputs; activations are bf16 here, so the bf16 tolerance applies."""
+    import mlx_rs_amd as m
+    rng = np.random.default_rng(0)
+    M, N, K = 32, 128, 128
+    scale = 1.0 / np.sqrt(K)
+    w = (rng.normal(0, 1, (K, N)) * scale).astype(np.float32)
+    x = orc.f32_to_bf16((rng.normal(0, 1, (M, K)) * scale).astype(np.float32))
+    q, s, b = orc.quantize(w, bits, 64)
+    y = m.ops.quantized_matmul(bf16_tensor(x, "cuda"), i32_tensor(q, "cuda"), bf16_tensor(s, "cuda"),
                                bf16_tensor(b, "cuda"), False, 64, bits)
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (M, N)
+    ref = f32_of_bits(x).astype(np.float64) @ orc.dequantize(q, s, b, bits, 64).astype(np.float64)
+    got = f32_of_bits(bits_u16(y)).astype(np.float64)
+    assert np.abs(got - ref).max() <= 2e-2 and np.linalg.norm(got - ref) / np.linalg.norm(ref) <= 1e-2
+    # gather form with three matrices and both index arrays; the oracle states the same identity
+    E = 3
+    wq = [orc.quantize((rng.normal(0, 1, (K, N)) * scale).astype(np.float32), bits, 64) for _ in range(E)]
+    W, S, B = (np.stack([t[i] for t in wq]) for i in range(3))
+    xs = orc.f32_to_bf16((rng.normal(0, 1, (5, 2, K)) * scale).astype(np.float32))
+    lhs, rhs = np.array([4, 0, 2, 2], np.uint32), np.array([2, 1, 0, 2], np.uint32)
+    yg = m.ops.gather_qmm(bf16_tensor(xs, "cuda"), i32_tensor(W, "cuda"), bf16_tensor(S, "cuda"), bf16_tensor(B, "cuda"),
+                          i32_tensor(lhs, "cuda"), i32_tensor(rhs, "cuda"), transpose=False, group_size=64, bits=bits)
+    torch.cuda.synchronize()
+    yo = orc.gather_qmm(xs, W, S, B, lhs, rhs, bits=bits, want="f32", transpose=False)
+    assert tuple(yg.shape) == yo.shape == (4, 2, N)
+    for j in range(4):
+        refj = f32_of_bits(xs[lhs[j]]).astype(np.float64) @ orc.dequantize(W[rhs[j]], S[rhs[j]], B[rhs[j]], bits, 64).astype(np.float64)
+        assert np.abs(yo[j] - refj).max() <= 1e-4
+    assert_close_bf16(bits_u16(yg), orc.f32_to_bf16(yo), what="gather_qmm, transpose = false")

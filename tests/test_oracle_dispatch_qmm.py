@@ -171,3 +171,30 @@ def test_strict_and_fused_rounding_points_stay_within_tolerance(orc):
     # thread count does not change a bit
     c, _ = orc.moe_forward(cfg, W, x, strict=True, n_threads=1)
     assert np.array_equal(a, c)
+
+
+def test_untransposed_gather_qmm_is_x_times_dequantized(orc):
+    """transpose = false (the layout of the reference's test_quantized_matmul,
+    mlx-rs/src/ops/quantization.rs:318-342): out = x @ dequantize(w), checked in float64, and on a
+    unit-scale integer case where every product and sum is exact."""
+    rng = np.random.default_rng(12)
+    M, N, K, E = 3, 128, 64, 2
+    for bits in (4, 8):
+        ws = [orc.quantize((rng.normal(0, 1, (K, N)) / 8).astype(np.float32), bits, 64) for _ in range(E)]
+        W, S, B = (np.stack([t[i] for t in ws]) for i in range(3))
+        x = orc.f32_to_bf16(rng.normal(0, 1, (4, M, K)).astype(np.float32))
+        lhs, rhs = np.array([3, 1], np.uint32), np.array([1, 0], np.uint32)
+        y = orc.gather_qmm(x, W, S, B, lhs, rhs, bits=bits, want="f32", transpose=False)
+        assert y.shape == (2, M, N)
+        for j in range(2):
+            ref = f32_of_bits(x[lhs[j]]).astype(np.float64) @ orc.dequantize(W[rhs[j]], S[rhs[j]], B[rhs[j]], bits, 64).astype(np.float64)
+            assert np.abs(y[j] - ref).max() <= 1e-4
+    # integers: codes 0..15 with scale 1, bias 0; x small integers: the result is the integer product
+    q = rng.integers(0, 16, (K, N)).astype(np.uint32)
+    packed = np.zeros((1, K, N // 8), np.uint32)
+    for c in range(8):
+        packed[0] |= q[:, c::8] << np.uint32(4 * c)
+    one, zero = orc.f32_to_bf16(np.ones((1, K, N // 64), np.float32)), orc.f32_to_bf16(np.zeros((1, K, N // 64), np.float32))
+    xi = rng.integers(-3, 4, (1, 2, K)).astype(np.float32)
+    y = orc.gather_qmm(orc.f32_to_bf16(xi), packed, one, zero, None, np.zeros(1, np.uint32), bits=4, want="f32", transpose=False)
+    assert np.array_equal(y[0], xi[0] @ q.astype(np.float32))

@@ -285,7 +285,11 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
   }
   mma(1);  // step nk - 1 (odd)
 
-  // ---- epilogue: D[i][j], lane holds column j = lane % 32 and rows 8 (r/4) + 4 (lane/32) + r%4.
+  // ---- epilogue: D[i][j], lane holds column j = lane % 32 and rows 8 (r/4) + 4 (lane/32) + r%4:
+  // stored from there, a wave's store instruction would write 2 bytes per lane (measured: 50 to
+  // 70 us per launch of the 256-row class at 4096 tokens, a third of the kernel).  Each wave turns
+  // its 32-row sub-tiles round in a private piece of LDS instead and stores 16 bytes per lane, whole
+  // 64- or 128-byte pieces of output rows.
   // perm_out: columns are written in the paired order within each 8-block (what a 4-bit
   // consumer of these rows expects as its activations).
   auto out_col = [&](int col) {
@@ -293,29 +297,49 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
     const int jj = col & 7;
     return (col & ~7) | (jj < 4 ? 2 * jj : 2 * (jj - 4) + 1);
   };
+  constexpr int CW = GLU ? 32 : 64;   // output columns of a wave
+  constexpr int ROWB = CW * 2 + 16;   // bytes per staged row (the 16 keep rows off each other's banks)
+  constexpr int CPR = CW / 8;         // 16-byte pieces per row
+  constexpr int RPI = 64 / CPR;       // rows one store instruction covers
+  static_assert(8 * 32 * ROWB <= large_lds_bytes(64), "staging does not fit the smallest tile's LDS");
+  __syncthreads();  // every wave has read its last operands: the space is free
+  unsigned char *const mine = lds_raw + wave * (32 * ROWB);
+  const int col0 = n0 + CW * wn;
+  const int my_piece = lane % CPR, my_row = lane / CPR;
+  const bool piece_ok = col0 + 8 * my_piece < N;  // N is a multiple of 16: a piece is inside or outside
 #pragma unroll
-  for (int m = 0; m < MS; ++m)
+  for (int m = 0; m < MS; ++m) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int tr = (BM / 2) * wm + 32 * m + 8 * (r >> 2) + 4 * kb + (r & 3);
-      if (tr < rows) {
-        const int64_t rr = row0 + tr;
-        const int64_t dst = a.dst_rows ? (int64_t)a.dst_rows[rr] : rr;
-        if constexpr (GLU) {
-          const int col = n0 + 32 * wn + ln;
-          if (col < N) {
-            const float g = acc[m][0][r], u = acc[m][1][r];
-            a.y[dst * N + out_col(col)] = (uint16_t)(cvt_pk_bf16(g / (1.0f + __expf(-g)) * u, 0.f) & 0xffffu);
-          }
-        } else {
+      const int row = 8 * (r >> 2) + 4 * kb + (r & 3);
+      if constexpr (GLU) {
+        const float g = acc[m][0][r], u = acc[m][1][r];
+        *reinterpret_cast<uint16_t *>(mine + row * ROWB + out_col(ln) * 2) = (uint16_t)(cvt_pk_bf16(g / (1.0f + __expf(-g)) * u, 0.f) & 0xffffu);
+      } else {
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const int col = n0 + 64 * wn + 32 * s + ln;
-            if (col < N) a.y[dst * N + out_col(col)] = (uint16_t)(cvt_pk_bf16(acc[m][s][r], 0.f) & 0xffffu);
-          }
-        }
+        for (int s = 0; s < 2; ++s)
+          *reinterpret_cast<uint16_t *>(mine + row * ROWB + out_col(32 * s + ln) * 2) = (uint16_t)(cvt_pk_bf16(acc[m][s][r], 0.f) & 0xffffu);
       }
     }
+    // LDS serves a wave's accesses in order; the fence and the barrier only pin the program order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int row = RPI * i + my_row;
+      const int tr = (BM / 2) * wm + 32 * m + row;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t *>(mine + row * ROWB + my_piece * 16);
+      if (tr < rows && piece_ok) {
+        const int64_t rr = row0 + tr;
+        const int64_t dst = a.dst_rows ? (int64_t)a.dst_rows[rr] : rr;
+        *reinterpret_cast<u32x4_t *>(a.y + dst * N + col0 + 8 * my_piece) = v;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
 }
 
 // Activation rows with every 8-block reordered to (x0,x4,x1,x5,x2,x6,x3,x7): the order in which

@@ -67,7 +67,7 @@ constexpr size_t large_lds_bytes(int bm) { return (size_t)2 * (bm + BR) * LDR * 
 // bound by that dequantisation, which is still far cheaper than streaming the weights once per
 // 8 tokens.
 template <int BITS, bool GLU, int MT>
-__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT == 4 ? 2 : 4))) void qmm_large_kernel(GroupedArgs a, const uint32_t *__restrict__ tiles, int n_ntiles) {
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT == 4 ? 2 : 4))) void qmm_large_kernel(GroupedArgs a, const uint32_t *__restrict__ tiles, int n_ntiles, int cap) {
   constexpr int NI = GLU ? 128 : 256;  // distinct output columns per block
   constexpr int BM = 64 * MT;          // token rows per block
   constexpr int NA = MT >= 2 ? MT / 2 : 1;  // 16-byte activation loads per thread and step
@@ -78,8 +78,9 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int nt = j % n_ntiles;
   const uint32_t mt_id = (uint32_t)(j / n_ntiles) * 8u + xcd;
+  // the record is fetched along with the count (index clamped to the list's capacity)
+  const uint4 rec = reinterpret_cast<const uint4 *>(tiles)[1 + (mt_id < (uint32_t)cap ? mt_id : (uint32_t)cap - 1u)];
   if (mt_id >= n_mtiles) return;
-  const uint4 rec = reinterpret_cast<const uint4 *>(tiles)[1 + mt_id];
   const int e = (int)rec.x;
   const int64_t row0 = rec.y;
   const int rows = (int)rec.z;
@@ -115,7 +116,11 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
   // B: thread covers 16 codes (half a K step) of weight row br; waves 0-3 / 4-7 hold gate / up
   const int br = tid >> 1, bh = tid & 1;
   const int mat = GLU ? (wave >> 2) : 0;  // wave-uniform
-  const int nrow = GLU ? n0 + (br & 127) : n0 + br;  // rows >= N read zeros through the descriptor
+  // paired output (columns of every 8-block in the order 0,4,1,5,2,6,3,7, what a 4-bit consumer
+  // of these rows expects as its activations): the thread at position p of an 8-block stages the
+  // weight row whose result belongs there, and the epilogue has nothing to permute
+  const int brp = a.y_paired ? ((br & ~7) | (((br & 7) >> 1) + ((br & 1) ? 4 : 0))) : br;
+  const int nrow = GLU ? n0 + (brp & 127) : n0 + brp;  // rows >= N read zeros through the descriptor
   const int64_t ebase = (int64_t)e * N;
   const __amdgpu_buffer_rsrc_t wr = make_rsrc((mat ? a.w1 : a.w0) + ebase * (row_bytes / 4), (uint32_t)N * row_bytes);
   const __amdgpu_buffer_rsrc_t sr = make_rsrc((mat ? a.s1 : a.s0) + ebase * gpr, (uint32_t)N * gpr * 2);
@@ -290,13 +295,6 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
   // 70 us per launch of the 256-row class at 4096 tokens, a third of the kernel).  Each wave turns
   // its 32-row sub-tiles round in a private piece of LDS instead and stores 16 bytes per lane, whole
   // 64- or 128-byte pieces of output rows.
-  // perm_out: columns are written in the paired order within each 8-block (what a 4-bit
-  // consumer of these rows expects as its activations).
-  auto out_col = [&](int col) {
-    if (!a.y_paired) return col;
-    const int jj = col & 7;
-    return (col & ~7) | (jj < 4 ? 2 * jj : 2 * (jj - 4) + 1);
-  };
   constexpr int CW = GLU ? 32 : 64;   // output columns of a wave
   constexpr int ROWB = CW * 2 + 16;   // bytes per staged row (the 16 keep rows off each other's banks)
   constexpr int CPR = CW / 8;         // 16-byte pieces per row
@@ -307,18 +305,38 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
   const int col0 = n0 + CW * wn;
   const int my_piece = lane % CPR, my_row = lane / CPR;
   const bool piece_ok = col0 + 8 * my_piece < N;  // N is a multiple of 16: a piece is inside or outside
+  // where the rows of this wave's half of the tile go: lane l fetches rows l and 64 + l of the
+  // half (one latency for all of them), a lane shuffle hands them out below
+  constexpr int NH = BM / 2 > 64 ? BM / 128 : 1;
+  uint32_t dst_half[NH];
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    int tr = (BM / 2) * wm + 64 * h + lane;
+    tr = tr < rows ? tr : rows - 1;
+    const int64_t rr = row0 + tr;
+    dst_half[h] = a.dst_rows ? a.dst_rows[rr] : (uint32_t)rr;
+  }
 #pragma unroll
   for (int m = 0; m < MS; ++m) {
+    // two rows of a column become one register (bf16 pair); neighbouring lanes (columns c, c + 1)
+    // swap halves, so that the even lane holds row r and the odd lane row r + 1 of both columns:
+    // one 4-byte LDS write per two results
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 8 * (r >> 2) + 4 * kb + (r & 3);
-      if constexpr (GLU) {
-        const float g = acc[m][0][r], u = acc[m][1][r];
-        *reinterpret_cast<uint16_t *>(mine + row * ROWB + out_col(ln) * 2) = (uint16_t)(cvt_pk_bf16(g / (1.0f + __expf(-g)) * u, 0.f) & 0xffffu);
-      } else {
+    for (int r = 0; r < 16; r += 2) {
+      const int row = 8 * (r >> 2) + 4 * kb + (r & 3) + (ln & 1);
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
-          *reinterpret_cast<uint16_t *>(mine + row * ROWB + out_col(32 * s + ln) * 2) = (uint16_t)(cvt_pk_bf16(acc[m][s][r], 0.f) & 0xffffu);
+      for (int s = 0; s < (GLU ? 1 : 2); ++s) {
+        uint32_t mine2;
+        if constexpr (GLU) {
+          const float g0 = acc[m][0][r], u0 = acc[m][1][r], g1 = acc[m][0][r + 1], u1 = acc[m][1][r + 1];
+          mine2 = cvt_pk_bf16(g0 / (1.0f + __expf(-g0)) * u0, g1 / (1.0f + __expf(-g1)) * u1);
+        } else {
+          mine2 = cvt_pk_bf16(acc[m][s][r], acc[m][s][r + 1]);
+        }
+        const uint32_t theirs = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine2, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+        // even lane: (mine.lo, theirs.lo) = row r, columns c, c + 1; odd: (theirs.hi, mine.hi) = row r + 1
+        const uint32_t both = __builtin_amdgcn_perm(theirs, mine2, (ln & 1) ? 0x03020706u : 0x05040100u);
+        *reinterpret_cast<uint32_t *>(mine + row * ROWB + (32 * s + (ln & ~1)) * 2) = both;
       }
     }
     // LDS serves a wave's accesses in order; the fence and the barrier only pin the program order
@@ -330,11 +348,9 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
       const int row = RPI * i + my_row;
       const int tr = (BM / 2) * wm + 32 * m + row;
       const u32x4_t v = *reinterpret_cast<const u32x4_t *>(mine + row * ROWB + my_piece * 16);
-      if (tr < rows && piece_ok) {
-        const int64_t rr = row0 + tr;
-        const int64_t dst = a.dst_rows ? (int64_t)a.dst_rows[rr] : rr;
-        *reinterpret_cast<u32x4_t *>(a.y + dst * N + col0 + 8 * my_piece) = v;
-      }
+      // row 32 m + row of the half is held by lane (32 m + row) % 64 of dst_half[(32 m + row) / 64]
+      const uint32_t dst = (uint32_t)__shfl((int)dst_half[(32 * m + RPI * i) >> 6], (32 * m + row) & 63, 64);
+      if (tr < rows && piece_ok) *reinterpret_cast<u32x4_t *>(a.y + (int64_t)dst * N + col0 + 8 * my_piece) = v;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -379,7 +395,7 @@ static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int ca
       return e;
     raised = true;
   }
-  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles);
+  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles, cap);
   return hipGetLastError();
 }
 

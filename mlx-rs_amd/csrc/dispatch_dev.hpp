@@ -230,4 +230,94 @@ __device__ __forceinline__ void dispatch_block(const uint32_t *flat, int64_t P, 
 
 constexpr int64_t kSingleMaxP = 4096;
 
+// The dispatch of at most 64 tokens whose k experts are distinct per token (what the selection
+// produces), by one block.  The stable order by pair index is then the order by token, and a
+// pair's place inside its expert's segment is the number of earlier tokens that chose the same
+// expert: it is read off a 64-bit token mask per expert.  Three barriers instead of the two dozen
+// of the general path; the same outputs bit for bit.
+// LDS (dynamic, passed in): 4 * E words.  P = T * k <= kSingleMaxP.
+constexpr int kMaskTokens = 64;
+__device__ __forceinline__ void dispatch_tokens_block(const uint32_t *flat, int T, int k, int E, uint32_t *lds,
+                                      uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
+                                      uint32_t *__restrict__ perm, uint32_t *__restrict__ inv_perm,
+                                      uint32_t *__restrict__ src_of, uint32_t *__restrict__ work) {
+  uint32_t *const mlo = lds, *const mhi = lds + E, *const off = lds + 2 * E, *const ridx = lds + 3 * E;
+  const int tid = threadIdx.x;
+  const int P = T * k;
+  constexpr int kPer = (int)(kSingleMaxP / kDispThreads);  // pairs per thread at most
+  for (int i = tid; i < 2 * E; i += kDispThreads) lds[i] = 0u;
+  __syncthreads();
+  uint32_t es[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int j = tid + i * kDispThreads;
+    es[i] = 0u;
+    if (j < P) {
+      uint32_t e = load_agent(flat + j);
+      e = e < (uint32_t)E ? e : (uint32_t)E - 1u;  // out-of-range ids are clamped, never written past LDS
+      es[i] = e;
+      const uint32_t t = (uint32_t)j / (uint32_t)k;
+      atomicOr(t < 32u ? &mlo[e] : &mhi[e], 1u << (t & 31u));
+    }
+  }
+  __syncthreads();
+  // wave 0: counts, their exclusive scan, one work record per expert with rows (ascending ids)
+  if (tid < kWave) {
+    uint32_t base = 0, n_active = 0;
+    for (int e0 = 0; e0 < E; e0 += kWave) {
+      const int e = e0 + tid;
+      const uint32_t c = e < E ? (uint32_t)(__popc(mlo[e]) + __popc(mhi[e])) : 0u;
+      uint32_t incl = c;
+      for (int d = 1; d < kWave; d <<= 1) {
+        const uint32_t v = __shfl_up(incl, d, kWave);
+        if (tid >= d) incl += v;
+      }
+      const uint32_t excl = base + incl - c;
+      const uint64_t bm = __ballot(c != 0u);
+      if (e < E) {
+        off[e] = excl;
+        if (counts) counts[e] = c;
+        if (offsets) offsets[e] = excl;
+        if (c != 0u) {
+          const uint32_t r = n_active + __popcll(bm & lanemask_lt());
+          ridx[e] = r;
+          if (work) {
+            uint32_t *rec = work + (size_t)r * kWorkWords;
+            rec[0] = (uint32_t)e;
+            rec[1] = excl;
+            rec[2] = c;
+            rec[3] = 1u;  // the source rows follow below
+          }
+        }
+      }
+      base += __shfl(incl, kWave - 1, kWave);
+      n_active += __popcll(bm);
+    }
+    if (tid == 0 && offsets) offsets[E] = base;
+    if (work)
+      for (int sl = (int)n_active + tid; sl < E; sl += kWave) {
+        work[(size_t)sl * kWorkWords + 2] = 0u;
+        work[(size_t)sl * kWorkWords + 3] = 0u;
+      }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int j = tid + i * kDispThreads;
+    if (j < P) {
+      const uint32_t e = es[i];
+      const uint32_t t = (uint32_t)j / (uint32_t)k;
+      const uint32_t lo = mlo[e], hi = mhi[e];
+      const uint32_t below = t < 32u ? (uint32_t)__popc(lo & ((1u << t) - 1u))
+                                     : (uint32_t)(__popc(lo) + __popc(hi & ((1u << (t - 32u)) - 1u)));
+      const uint32_t pos = off[e] + below;
+      perm[pos] = (uint32_t)j;
+      if (inv_perm) inv_perm[j] = pos;
+      if (src_of) src_of[pos] = t;
+      // source rows of the first rows of every segment, so that a consumer needs one load
+      if (work && below < (uint32_t)kWorkSrc) work[(size_t)ridx[e] * kWorkWords + 4 + below] = t;
+    }
+  }
+}
+
 }  // namespace mi_moe

@@ -71,8 +71,13 @@ __global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
   if (!last) return;
 
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  dispatch_block(topk_idx, (int64_t)T * k, E, nbits, k, lds, counts, offsets, perm, inv_perm, src_of,
-                 work, mtiles, cap256, big_thr);
+  // at most 64 tokens, distinct experts per token: the mask form of the dispatch (the tiled lists
+  // belong to batches far above this kernel's, the host passes none)
+  if (mtiles == nullptr && T <= kMaskTokens)
+    dispatch_tokens_block(topk_idx, T, k, E, lds, counts, offsets, perm, inv_perm, src_of, work);
+  else
+    dispatch_block(topk_idx, (int64_t)T * k, E, nbits, k, lds, counts, offsets, perm, inv_perm, src_of,
+                   work, mtiles, cap256, big_thr);
 }
 
 bool router_fused_applies(int64_t T, int E, int k) {

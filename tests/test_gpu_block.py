@@ -76,13 +76,18 @@ def test_fused_router_equals_the_separate_kernels(orc):
     entry points run them as separate kernels.  Same integers and scores, call after call (the
     launch leaves its arrival counters at zero), across batch sizes on both sides of the switch."""
     import mlx_rs_amd as m
-    H, E, k, I = 256, 128, 8, 128
+    _fused_vs_separate(orc, m, 256, 128, 8, 128, [1, 64, 3, 64, 17, 65, 2, 40, 1])
+    # more pairs than the dispatching workgroup has threads (60 x 20 = 1200), few experts
+    _fused_vs_separate(orc, m, 128, 32, 20, 128, [60, 33, 64])
+
+
+def _fused_vs_separate(orc, m, H, E, k, I, batches):
     W = host_layer(orc, H, E, k, I, 4, 21, zipf_s=0.7)
     blk = device_block(m, m.MoeConfig(H, E, k, I), W)
     rw = bf16_tensor(W["router_w"], "cuda")
     rb = torch.from_numpy(W["router_bias"]).cuda()
-    for rep, T in enumerate([1, 64, 3, 64, 17, 65, 2, 40, 1]):
-        print(f"fused router T={T}", flush=True)
+    for rep, T in enumerate(batches):
+        print(f"fused router H={H} E={E} k={k} T={T}", flush=True)
         x = bf16_tensor(host_tokens(orc, T, H, 100 + rep), "cuda")
         _, dbg = blk.forward(x, debug=True)
         inds, sc = m.ops.route(x, rw, k, 0, router_bias=rb)

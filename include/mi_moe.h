@@ -26,8 +26,11 @@
  *    a time (MLX itself is not thread safe, .github/workflows/validate.yml:46), and
  *    forwards through one handle must not overlap on the GPU (use one stream per handle):
  *    a handle owns 260 bytes of device memory (arrival counters of the decode router
- *    kernel), allocated by mi_moe_create on the current device and freed by
- *    mi_moe_destroy.  No other entry point allocates device memory.
+ *    kernel) and three streams with four events (default priority; a forward of 192 tokens
+ *    or more forks its independent kernel chains onto them from `stream` and joins them
+ *    back before it returns, which is also what a graph capture of `stream` records), all
+ *    created by mi_moe_create on the current device and released by mi_moe_destroy.  No
+ *    other entry point allocates device memory or creates streams.
  *
  * Weight format = MLX "affine" quantisation (mlx-rs/src/ops/quantization.rs:31-47,
  * 85-87, 306-309): element c of a row lives in uint32 word c/(32/bits) at bit

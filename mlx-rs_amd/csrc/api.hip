@@ -128,7 +128,23 @@ struct mi_moe_s {
   mi_moe_config cfg;
   mi_moe_weights w;
   uint32_t *counters = nullptr;  // device: arrival counters of the fused decode router, zero at rest
+  // prefill-sized batches: the tile classes and the streamed segments are independent chains
+  // (gate/up then down over the same rows); three of the four run on these streams, forked from
+  // and joined back into the caller's stream by events
+  hipStream_t side[3] = {nullptr, nullptr, nullptr};
+  hipEvent_t fork = nullptr, join[3] = {nullptr, nullptr, nullptr};
 };
+
+void destroy_handle(mi_moe_s *h) {
+  if (!h) return;
+  if (h->counters) (void)hipFree(h->counters);
+  for (int i = 0; i < 3; ++i) {
+    if (h->side[i]) (void)hipStreamDestroy(h->side[i]);
+    if (h->join[i]) (void)hipEventDestroy(h->join[i]);
+  }
+  if (h->fork) (void)hipEventDestroy(h->fork);
+  delete h;
+}
 
 extern "C" {
 
@@ -160,18 +176,22 @@ int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_mo
   const size_t cbytes = (size_t)(1 + kFusedRouterMaxTokens) * sizeof(uint32_t);
   hipError_t e = hipMalloc(reinterpret_cast<void **>(&h->counters), cbytes);
   if (e == hipSuccess) e = hipMemset(h->counters, 0, cbytes);
+  // streams (default priority) and events for the independent chains of a prefill-sized forward
+  for (int i = 0; i < 3 && e == hipSuccess; ++i) {
+    e = hipStreamCreateWithFlags(&h->side[i], hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&h->join[i], hipEventDisableTiming);
+  }
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&h->fork, hipEventDisableTiming);
   if (e != hipSuccess) {
-    if (h->counters) (void)hipFree(h->counters);
-    delete h;
-    return fail("create: device memory for the handle: %s", hipGetErrorString(e));
+    destroy_handle(h);
+    return fail("create: device memory, streams and events of the handle: %s", hipGetErrorString(e));
   }
   *out = h;
   return 0;
 }
 
 int mi_moe_destroy(mi_moe_handle h) {
-  if (h && h->counters) (void)hipFree(h->counters);
-  delete h;
+  destroy_handle(h);
   return 0;
 }
 
@@ -262,23 +282,47 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   a.y = f.hh;
   a.N = c.intermediate;
   a.K = c.hidden;
-  MI_HIP(launch_grouped_qmm(a, true, st));
-  MI_STAGE_DONE();
   // down: rows read in sorted order, written back in (token, slot) order
-  a.x = f.hh;
-  a.x_perm = f.hh;
-  a.x_paired = paired;
-  a.y_paired = false;
-  a.src_rows = nullptr;
-  a.src_in_work = false;
-  a.dst_rows = f.perm;
-  a.w0 = h->w.down.w; a.s0 = h->w.down.scales; a.b0 = h->w.down.biases;
-  a.w1 = nullptr; a.s1 = a.b1 = nullptr;
-  a.y = f.y;
-  a.N = c.hidden;
-  a.K = c.intermediate;
-  MI_HIP(launch_grouped_qmm(a, false, st));
-  MI_STAGE_DONE();
+  GroupedArgs d = a;
+  d.x = f.hh;
+  d.x_perm = f.hh;
+  d.x_paired = paired;
+  d.y_paired = false;
+  d.src_rows = nullptr;
+  d.src_in_work = false;
+  d.dst_rows = f.perm;
+  d.w0 = h->w.down.w; d.s0 = h->w.down.scales; d.b0 = h->w.down.biases;
+  d.w1 = nullptr; d.s1 = d.b1 = nullptr;
+  d.y = f.y;
+  d.N = c.hidden;
+  d.K = c.intermediate;
+  if (large_qmm_applies(a) && !ev) {
+    // Four chains that share no rows: the three tile classes and the streamed segments, each
+    // gate/up then down.  The short classes leave most of the chip idle when they run alone
+    // (a few dozen workgroups of 64 K steps each); side by side they fill it.  The longest chain
+    // stays on the caller's stream.
+    MI_HIP(hipEventRecord(h->fork, st));
+    for (int i = 0; i < 3; ++i) MI_HIP(hipStreamWaitEvent(h->side[i], h->fork, 0));
+    for (int chain = 0; chain < 4; ++chain) {
+      hipStream_t s = chain == 0 ? st : h->side[chain - 1];
+      if (chain < 3) {
+        MI_HIP(launch_large_qmm_class(a, true, chain, s));
+        MI_HIP(launch_large_qmm_class(d, false, chain, s));
+      } else {
+        MI_HIP(launch_small_qmm(a, true, s));
+        MI_HIP(launch_small_qmm(d, false, s));
+      }
+    }
+    for (int i = 0; i < 3; ++i) {
+      MI_HIP(hipEventRecord(h->join[i], h->side[i]));
+      MI_HIP(hipStreamWaitEvent(st, h->join[i], 0));
+    }
+  } else {
+    MI_HIP(launch_grouped_qmm(a, true, st));
+    MI_STAGE_DONE();
+    MI_HIP(launch_grouped_qmm(d, false, st));
+    MI_STAGE_DONE();
+  }
   MI_HIP(launch_combine(f.y, f.topk_w, nullptr, T, c.top_k, c.hidden, norm_weight ? x_in : nullptr, out, st));
   MI_STAGE_DONE();
 #undef MI_STAGE_DONE

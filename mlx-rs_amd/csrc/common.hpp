@@ -193,6 +193,11 @@ hipError_t launch_router_fused(const uint16_t *x, const uint16_t *wg, const floa
                                int big_thr, hipStream_t st);
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
+// the same work in its independent parts: one tile class (0, 1, 2 = 256-, 128-, 64-row tiles) of
+// the tiled kernel, or the streaming kernel alone.  No part reads what another one writes.
+bool large_qmm_applies(const GroupedArgs &a);
+hipError_t launch_large_qmm_class(const GroupedArgs &a, bool glu, int cls, hipStream_t st);
+hipError_t launch_small_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *out, hipStream_t st);
 hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,

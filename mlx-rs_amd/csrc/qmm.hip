@@ -437,10 +437,9 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   else qmm_small_kernel<BITS, GLU, 1><<<grid, 256, lds, st>>>(a, tt);
 }
 
-hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
+// the streaming kernel on its own: segments the dispatch did not list as M tiles
+hipError_t launch_small_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
   if (a.max_active <= 0 || a.total_rows <= 0) return hipSuccess;
-  // long segments (listed as M tiles by the dispatch) go to the tiled kernel, the rest below
-  if (hipError_t e = launch_large_qmm(a, glu, st); e != hipSuccess) return e;
   if (a.bits == 4) {
     if (glu) launch_small<4, true>(a, st);
     else launch_small<4, false>(a, st);
@@ -449,6 +448,13 @@ hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
     else launch_small<8, false>(a, st);
   }
   return hipGetLastError();
+}
+
+hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
+  if (a.max_active <= 0 || a.total_rows <= 0) return hipSuccess;
+  // long segments (listed as M tiles by the dispatch) go to the tiled kernel, the rest below
+  if (hipError_t e = launch_large_qmm(a, glu, st); e != hipSuccess) return e;
+  return launch_small_qmm(a, glu, st);
 }
 
 }  // namespace mi_moe

@@ -399,21 +399,28 @@ static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int ca
   return hipGetLastError();
 }
 
+// class 0 / 1 / 2 = the 256- / 128- / 64-row tile list.  A segment is at most max_rows_per_expert
+// long: a class that cannot occur is not launched.
 template <int BITS, bool GLU>
-static hipError_t launch_classes(const GroupedArgs &a, hipStream_t st) {
-  // a segment is at most max_rows_per_expert long: classes that cannot occur are not launched
-  const int cap_small = a.tile_cap_e;
-  if (a.max_rows_per_expert > 128)
-    if (hipError_t e = launch_one<BITS, GLU, 4>(a, tile_list(a.mtiles, 0, a.max_mtiles, a.tile_cap_e), a.max_mtiles, st); e != hipSuccess) return e;
-  if (a.max_rows_per_expert > 64)
-    if (hipError_t e = launch_one<BITS, GLU, 2>(a, tile_list(a.mtiles, 1, a.max_mtiles, a.tile_cap_e), cap_small, st); e != hipSuccess) return e;
-  return launch_one<BITS, GLU, 1>(a, tile_list(a.mtiles, 2, a.max_mtiles, a.tile_cap_e), cap_small, st);
+static hipError_t launch_class(const GroupedArgs &a, int cls, hipStream_t st) {
+  const uint32_t *const list = tile_list(a.mtiles, cls, a.max_mtiles, a.tile_cap_e);
+  if (cls == 0) return a.max_rows_per_expert > 128 ? launch_one<BITS, GLU, 4>(a, list, a.max_mtiles, st) : hipSuccess;
+  if (cls == 1) return a.max_rows_per_expert > 64 ? launch_one<BITS, GLU, 2>(a, list, a.tile_cap_e, st) : hipSuccess;
+  return launch_one<BITS, GLU, 1>(a, list, a.tile_cap_e, st);
+}
+
+bool large_qmm_applies(const GroupedArgs &a) { return a.mtiles && a.tile_cap_e > 0 && a.x_perm; }
+
+hipError_t launch_large_qmm_class(const GroupedArgs &a, bool glu, int cls, hipStream_t st) {
+  if (!large_qmm_applies(a)) return hipSuccess;
+  if (a.bits == 4) return glu ? launch_class<4, true>(a, cls, st) : launch_class<4, false>(a, cls, st);
+  return glu ? launch_class<8, true>(a, cls, st) : launch_class<8, false>(a, cls, st);
 }
 
 hipError_t launch_large_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
-  if (!a.mtiles || a.tile_cap_e <= 0 || !a.x_perm) return hipSuccess;
-  if (a.bits == 4) return glu ? launch_classes<4, true>(a, st) : launch_classes<4, false>(a, st);
-  return glu ? launch_classes<8, true>(a, st) : launch_classes<8, false>(a, st);
+  for (int cls = 0; cls < 3; ++cls)
+    if (hipError_t e = launch_large_qmm_class(a, glu, cls, st); e != hipSuccess) return e;
+  return hipSuccess;
 }
 
 }  // namespace mi_moe

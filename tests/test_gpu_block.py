@@ -174,11 +174,14 @@ def test_graph_replays_equal_eager(orc, T):
         torch.cuda.synchronize()
 
 
-def test_two_handles_on_two_streams(orc):
+@pytest.mark.parametrize("T", [16, 400])
+def test_two_handles_on_two_streams(orc, T):
     """Handles are independent: two layers running concurrently on two streams (each with its own
-    workspace) give what they give one after the other."""
+    workspace) give what they give one after the other.  At 400 tokens each forward also forks its
+    kernel chains onto the handle's own streams and joins them back."""
     import mlx_rs_amd as m
-    H, E, k, I, T = 256, 16, 4, 256, 16
+    H, E, k, I = 256, 16, 4, 256
+    print(f"two handles T={T}", flush=True)
     blks, xs, refs = [], [], []
     for i in range(2):
         W = host_layer(orc, H, E, k, I, 4, seed=90 + i)

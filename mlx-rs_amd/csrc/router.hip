@@ -116,15 +116,26 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
 #pragma unroll
     for (int b = 0; b < 2; ++b) acc[a][b] = f64x4_t{0.0, 0.0, 0.0, 0.0};
 
-  for (int c = wave; c < H / 32; c += 4) {
-    uint32_t xa[2][4], wb[2][4];
+  // Two register sets take turns: the loads of the next chunk are issued before the current
+  // chunk is multiplied and waited for after it.  (Every load is unconditional, its index clamped
+  // and opaque: a load under a condition makes the compiler wait for all loads in flight, and a
+  // transparent index lets it fold the prefetch back into the next iteration's top.)
+  const int nchunks = H / 32;
+  struct Chunk {
+    uint4 x[2], w[2];
+  };
+  auto fetch = [&](int c, Chunk &R) __attribute__((always_inline)) {
+    int cc = c < nchunks ? c : nchunks - 1;
+    asm volatile("" : "+s"(cc));
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
-      const uint4 v = *reinterpret_cast<const uint4 *>(xr[a] + c * 32);
-      const uint4 u = *reinterpret_cast<const uint4 *>(wr[a] + c * 32);
-      xa[a][0] = v.x; xa[a][1] = v.y; xa[a][2] = v.z; xa[a][3] = v.w;
-      wb[a][0] = u.x; wb[a][1] = u.y; wb[a][2] = u.z; wb[a][3] = u.w;
+      R.x[a] = *reinterpret_cast<const uint4 *>(xr[a] + cc * 32);
+      R.w[a] = *reinterpret_cast<const uint4 *>(wr[a] + cc * 32);
     }
+  };
+  auto multiply = [&](const Chunk &R) __attribute__((always_inline)) {
+    const uint32_t xa[2][4] = {{R.x[0].x, R.x[0].y, R.x[0].z, R.x[0].w}, {R.x[1].x, R.x[1].y, R.x[1].z, R.x[1].w}};
+    const uint32_t wb[2][4] = {{R.w[0].x, R.w[0].y, R.w[0].z, R.w[0].w}, {R.w[1].x, R.w[1].y, R.w[1].z, R.w[1].w}};
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       double av[2], bv[2];
@@ -139,7 +150,21 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
         for (int b = 0; b < 2; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[a], bv[b], acc[a][b], 0, 0, 0);
     }
+  };
+  Chunk r0, r1;
+  fetch(wave, r0);
+  int c = wave;
+  for (; c + 4 < nchunks; c += 8) {  // two chunks per turn, both multiplied without a condition
+    fetch(c + 4, r1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(r0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(c + 8, r0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(r1);
+    __builtin_amdgcn_sched_barrier(0);
   }
+  if (c < nchunks) multiply(r0);  // an odd chunk left over (already fetched)
 
   __shared__ double part[4][4][4][64];  // [wave][tile][r][lane]
 #pragma unroll

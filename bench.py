@@ -39,6 +39,9 @@ def parse():
     ap.add_argument("--layers", type=int, default=0, help="distinct weight sets to rotate over (0 = auto)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--serial-kernels", action="store_true",
+                    help="every step through mi_moe_forward_timed: kernels run one after the other on one stream "
+                         "(for per-kernel profiles; a prefill-sized mi_moe_forward runs four chains side by side)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only-headline", action="store_true", help="run only the headline batch of the workload")
     ap.add_argument("--batches", default="", help="comma-separated batch sizes to run besides the headline batch")
@@ -122,8 +125,12 @@ def main():
             counts_stats.append((int(c.max()), float(c.mean()), int(c.min())))
         n_active = sum(actives) / len(actives)
 
+        if args.serial_kernels:
+            step_fn = lambda blk, xx, oo: blk.forward_timed(xx, out=oo)
+        else:
+            step_fn = lambda blk, xx, oo: blk.forward(xx, out=oo)
         graph = None
-        if not args.no_graph:
+        if not args.no_graph and not args.serial_kernels:
             # one graph replays a forward through every weight set (launch overhead amortised the
             # way a serving loop would capture a whole decode step)
             s = torch.cuda.Stream()
@@ -150,10 +157,10 @@ def main():
             ms = time_steps(lambda i: graph.replay(), reps, wreps, torch) / n_layers
             steps_done = reps * n_layers
         else:
-            ms = time_steps(lambda i: blocks[i % n_layers].forward(x, out=outs[i % n_layers]),
+            ms = time_steps(lambda i: step_fn(blocks[i % n_layers], x, outs[i % n_layers]),
                             args.steps, args.warmup, torch)
             steps_done = args.steps
-        eager_ms = time_steps(lambda i: blocks[i % n_layers].forward(x, out=outs[i % n_layers]),
+        eager_ms = time_steps(lambda i: step_fn(blocks[i % n_layers], x, outs[i % n_layers]),
                               args.steps, args.warmup, torch)
 
         # spread of single steps (event pair around each eager step) and the cache-resident figure
@@ -161,12 +168,12 @@ def main():
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
         for i, (e0, e1) in enumerate(evs):
             e0.record()
-            blocks[i % n_layers].forward(x, out=outs[i % n_layers])
+            step_fn(blocks[i % n_layers], x, outs[i % n_layers])
             e1.record()
         torch.cuda.synchronize()
         per_step = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
         pct = lambda q: per_step[min(len(per_step) - 1, int(q * len(per_step)))]
-        resident_ms = time_steps(lambda i: blocks[0].forward(x, out=outs[0]), args.steps, args.warmup, torch)
+        resident_ms = time_steps(lambda i: step_fn(blocks[0], x, outs[0]), args.steps, args.warmup, torch)
 
         # per-kernel durations from HIP events on the launch stream, same K steps
         stage = [0.0] * m.capi.N_STAGES
@@ -227,7 +234,7 @@ def main():
         "config": {"workload": "%s %s-bit g64 MoE layer, %s, batch %d" % (cfg_name, cfg.bits, args.workload, headline),
                    "hidden": cfg.hidden, "n_experts": cfg.n_experts, "top_k": cfg.top_k,
                    "intermediate": cfg.intermediate, "bits": cfg.bits, "batch": headline,
-                   "weight_sets_rotated": n_layers, "launch": "eager" if args.no_graph else "hip-graph"},
+                   "weight_sets_rotated": n_layers, "launch": "eager, one kernel at a time" if args.serial_kernels else ("eager" if args.no_graph else "hip-graph")},
         "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
     }
     print(json.dumps(out))

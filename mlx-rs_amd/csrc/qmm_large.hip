@@ -17,6 +17,8 @@
 // Three K steps of global loads are in flight while the current one is multiplied.
 #include <type_traits>
 
+#include <atomic>
+
 #include "common.hpp"
 
 #ifndef MI_MOE_WEAVE
@@ -386,14 +388,18 @@ static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int ca
   const int n_ntiles = (a.N + ni - 1) / ni;
   const unsigned grid = (unsigned)((cap + 7) / 8) * 8u * (unsigned)n_ntiles;
   constexpr size_t lds = large_lds_bytes(64 * MT);
-  // more LDS per block than a kernel gets without asking
-  static bool raised = false;
-  if (!raised) {
+  // more LDS per block than a kernel gets without asking: asked for once per device (the attribute
+  // belongs to the device's copy of the kernel); two threads asking at once is harmless
+  constexpr int kMaxDevices = 64;
+  static std::atomic<bool> raised[kMaxDevices];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices || !raised[dev].load(std::memory_order_acquire)) {
     if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<BITS, GLU, MT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         e != hipSuccess)
       return e;
-    raised = true;
+    if (dev >= 0 && dev < kMaxDevices) raised[dev].store(true, std::memory_order_release);
   }
   qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles, cap);
   return hipGetLastError();

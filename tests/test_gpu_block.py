@@ -198,3 +198,24 @@ def test_two_handles_on_two_streams(orc, T):
     torch.cuda.synchronize()
     for i in range(2):
         assert torch.equal(outs[i].view(torch.int16), refs[i].view(torch.int16)), f"handle {i}"
+
+
+def test_empty_batch_and_leading_axes(orc):
+    """[B, L, H] goes through as B*L rows (the Module contract, mlx-rs/src/module/module.rs:28-50,
+    as the dense Mlp is called with [B, L, H], mlx-lm/src/models/qwen3.rs:321-324); an empty batch
+    succeeds and touches nothing."""
+    import mlx_rs_amd as m
+    H, E, k, I = 256, 8, 2, 512
+    W = host_layer(orc, H, E, k, I, 4, seed=5)
+    blk = device_block(m, m.MoeConfig(H, E, k, I), W)
+    x = bf16_tensor(host_tokens(orc, 6, H, seed=6), "cuda")
+    flat = blk.forward(x).clone()
+    cube = blk.forward(x.reshape(2, 3, H))
+    torch.cuda.synchronize()
+    assert cube.shape == (2, 3, H)
+    assert torch.equal(cube.reshape(6, H).view(torch.int16), flat.view(torch.int16))
+    empty = blk.forward(x[:0])
+    torch.cuda.synchronize()
+    assert empty.shape == (0, H)
+    out, dbg = blk.forward(x[:0].reshape(0, 1, H), debug=True)
+    assert out.shape == (0, 1, H) and dbg["perm"].numel() == 0

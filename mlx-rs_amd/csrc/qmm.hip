@@ -81,6 +81,9 @@ extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
 #ifndef MI_MOE_RING
 #define MI_MOE_RING 4
 #endif
+#ifndef MI_MOE_PRECISE_BELOW
+#define MI_MOE_PRECISE_BELOW 2  // blocks per CU up to which the ring takes the unconditional form
+#endif
 
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 
@@ -104,14 +107,22 @@ struct ChunkRegs {
 // xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
 __host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
 __host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }  // 16 rows x K/64 bf16
-__host__ __device__ constexpr size_t small_lds_bytes(int K, int tt, int TT, int n_tensors) {
-  return (size_t)(tt + 1) * x_stride_bytes(K) + (size_t)(K / 64) * TT * 4 +
+// sk: K values of the activation rows staged at a time (a slab; the whole row when sk = K)
+__host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors) {
+  return (size_t)(tt + 1) * x_stride_bytes(sk) + (size_t)(sk / 64) * TT * 4 +
          (size_t)4 * n_tensors * sb_tile_bytes(K);
 }
 
-template <int BITS, bool GLU, int KW>
+// PRECISE: the ring's refills are issued without a condition (chunk index clamped), so the compiler
+// waits for exactly the chunk it needs and a wave really keeps D chunks in flight.  With the
+// conditional refills it waits for every load in flight before each chunk; that is the faster form
+// (by 2-3 %) when 16 and more waves share a CU, and several times slower when long rows leave
+// room for two blocks per CU only (K = 4096: 8 KB of LDS per staged token).
+// SLABS: the activation rows are staged sk K values at a time (rows too long for LDS); without it
+// sk = K and the slab loop below is a single pass the compiler folds away.
+template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8)))
-void qmm_small_kernel(GroupedArgs a, int tt) {
+void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   constexpr int NW = 4 / KW;                    // row tiles per block
   constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one 16-byte load per lane)
   constexpr int XV = BITS == 4 ? 4 : 2;         // 16-byte pieces of activations per lane per chunk
@@ -171,8 +182,10 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
   // the weight stream does not depend on the tokens: start it before anything else
   Regs ring[D];
 #pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (ch0 + d < ch1) issue(ch0 + d, ring[d]);
+  for (int d = 0; d < D; ++d) {
+    if constexpr (PRECISE) issue(ch0 + d < nchunks ? ch0 + d : nchunks - 1, ring[d]);
+    else if (ch0 + d < ch1) issue(ch0 + d, ring[d]);
+  }
 
   // scales and biases of the wave's 16 rows: K/2 contiguous bytes per tensor, fetched with
   // fully coalesced 16-byte loads now and parked in LDS (wave-private) before the chunk loop
@@ -188,13 +201,17 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
         sbv[t][i] = __builtin_amdgcn_raw_buffer_load_b128((t & 1) ? br[t >> 1] : sr[t >> 1], sb_goff, i * 1024, 0);
 
   MI_STAMP(1);
-  const int xstride = x_stride_bytes(K);
+  // Long rows are staged a slab of sk K values at a time (sk = K: the whole row); the weight
+  // stream, its ring and the accumulators run on across the slabs.
+  const int sk = SLABS ? sk_arg : K;
+  const int xstride = x_stride_bytes(sk);
+  const int groups_per_slab = sk / 64;
   const uint32_t nib_mask = opaque_reg(0x000f000fu), nib_magic = opaque_reg(0x43004300u);  // q -> bf16 128 + q
 
   extern __shared__ __align__(16) unsigned char lds[];
   unsigned char *lds_x = lds;
-  float *lds_gs = reinterpret_cast<float *>(lds + (tt + 1) * xstride);  // [groups][TT] sums of x
-  unsigned char *lds_sb = lds + (tt + 1) * xstride + groups_per_row * TT * 4 + wave * NTEN * sbt;
+  float *lds_gs = reinterpret_cast<float *>(lds + (tt + 1) * xstride);  // [groups of the slab][TT] sums of x
+  unsigned char *lds_sb = lds + (tt + 1) * xstride + groups_per_slab * TT * 4 + wave * NTEN * sbt;
 
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait)
 #pragma unroll
@@ -214,84 +231,23 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
   // zero row and zero group sums (slots that carry no token stay zero for the whole launch)
   for (int i = threadIdx.x; i < xstride / 16; i += 256)
     *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
-  for (int i = threadIdx.x; i < groups_per_row * TT / 4; i += 256)
+  for (int i = threadIdx.x; i < groups_per_slab * TT / 4; i += 256)
     *reinterpret_cast<uint4 *>(lds_gs + i * 4) = make_uint4(0, 0, 0, 0);
 
   for (int t0 = 0; t0 < cnt; t0 += tt) {
     const int nt = cnt - t0 < tt ? cnt - t0 : tt;  // tokens of this tile
-    __syncthreads();  // zero fill done / every wave is done reading the previous tile
-    if (t0 > 0) {
-#pragma unroll
-      for (int d = 0; d < D; ++d)
-        if (ch0 + d < ch1) issue(ch0 + d, ring[d]);
-    }
-    // stage the tile's activation rows in LDS (4-bit: each 8-block stored as the pairs
-    // (x0,x4)(x1,x5)(x2,x6)(x3,x7) the nibble unpacking produces) and the per-group sums of x.
-    // Rows past nt are never read (their lanes read the zero row); their group sums are cleared.
-    if (t0 > 0 && nt < tt)
-      for (int i = threadIdx.x; i < (tt - nt) * groups_per_row; i += 256)
-        lds_gs[(i / (tt - nt)) * TT + nt + i % (tt - nt)] = 0.f;
-    // wave w stages token slots w, w+4, ...: the source row is wave-uniform (read from the
-    // record through the scalar cache) and every load of a row is issued before the first use
-    for (int ts = wave; ts < nt; ts += 4) {
-      const int64_t r = r0 + t0 + ts;
-      int64_t src = r;
-      if (rec_src && t0 + ts < 12) src = a.work[(size_t)blockIdx.y * 16 + 4 + t0 + ts];
-      else if (a.src_rows) src = a.src_rows[r];
-      const uint16_t *xr = a.x + src * K;
-      for (int b0 = 0; b0 < K / 8; b0 += 256) {
-        uint4 v[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int blk = b0 + j * 64 + lane;
-          v[j] = make_uint4(0, 0, 0, 0);
-          if (blk < K / 8) v[j] = *reinterpret_cast<const uint4 *>(xr + blk * 8);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int blk = b0 + j * 64 + lane;
-          const uint4 w = v[j];
-          float sum = ((bf16lo_to_f32(w.x) + bf16hi_to_f32(w.x)) + (bf16lo_to_f32(w.y) + bf16hi_to_f32(w.y))) +
-                      ((bf16lo_to_f32(w.z) + bf16hi_to_f32(w.z)) + (bf16lo_to_f32(w.w) + bf16hi_to_f32(w.w)));
-          sum += __shfl_xor(sum, 1, kWave);
-          sum += __shfl_xor(sum, 2, kWave);
-          sum += __shfl_xor(sum, 4, kWave);
-          if (blk < K / 8) {
-            uint4 p = w;
-            if (BITS == 4 && !a.x_paired) {
-              p.x = (w.x & 0xffffu) | (w.z << 16);
-              p.y = (w.x >> 16) | (w.z & 0xffff0000u);
-              p.z = (w.y & 0xffffu) | (w.w << 16);
-              p.w = (w.y >> 16) | (w.w & 0xffff0000u);
-            }
-            *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = p;
-            if ((blk & 7) == 0) lds_gs[(blk >> 3) * TT + ts] = sum;
-          }
-        }
-      }
-    }
-    MI_STAMP(2);
-    __syncthreads();
-    MI_STAMP(3);
 
-    // activation row of this lane (A operand); lanes without data read the zero row
-    const int ts = BITS == 4 ? (c & 7) : c;
-    bool a_on = ts < nt;
-    if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
-    const unsigned char *xl = lds_x + (a_on ? ts : tt) * xstride + kb * (CH / 4) * 2;
-
+    // set after a slab has been staged (kept out of the staging's way: they cost registers there)
+    const unsigned char *xl;  // activation row of this lane (A operand)
+    const float *gsl;         // group sums of x for this lane's 4 D rows (token slots), first group of the slab
     f32x4_t tot[NM];
-#pragma unroll
-    for (int m = 0; m < NM; ++m) tot[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    // group sums of x for this lane's 4 D rows (token slots), first group of chunk 0
-    const float *gsl = lds_gs + (BITS == 4 ? (kb >> 1) * TT + 4 * (kb & 1) : 4 * kb);
+    int slab_ch0 = 0;  // first chunk of the slab that is in LDS
 
     // one chunk: MFMAs on raw codes, then scale and bias applied to the fp32 group sums
     auto compute = [&](int ch, const Regs &R) {
       uint4 xv[XV];
 #pragma unroll
-      for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl + ch * CH * 2 + i * 16);
+      for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl + (SLABS ? ch - slab_ch0 : ch) * CH * 2 + i * 16);
       f32x4_t acc[NM];
 #pragma unroll
       for (int m = 0; m < NM; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -331,7 +287,7 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
         }
       }
       // sum_c x_c (s (128 + q_c - 128) + b) = s * acc + (b - 128 s) * sum_c x_c   (8-bit: no offset)
-      const float4 xs = *reinterpret_cast<const float4 *>(gsl + ch * (BITS == 4 ? 2 : 1) * TT);
+      const float4 xs = *reinterpret_cast<const float4 *>(gsl + (SLABS ? ch - slab_ch0 : ch) * (BITS == 4 ? 2 : 1) * TT);
 #pragma unroll
       for (int m = 0; m < NM; ++m) {
         const int goff = ch * (BITS == 4 ? 4 : 2);
@@ -345,18 +301,131 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
       }
     };
 
-    MI_STAMP(4);
-    // D chunks in flight: slot d is refilled as soon as its chunk has been consumed.  (Issuing the
-    // refills without a condition, so that the compiler waits per slot instead of for all loads in
-    // flight, was measured 2-3 % slower here: enough waves are resident to cover the wait.)
-    for (int base = ch0; base < ch1; base += D) {
+
+    // staging of the K values [s0, s0 + sl) of the tile's rows
+    auto stage_rows = [&](int s0, int sl) __attribute__((always_inline)) {
+      // stage the slab of the tile's activation rows in LDS (4-bit: each 8-block stored as the pairs
+      // (x0,x4)(x1,x5)(x2,x6)(x3,x7) the nibble unpacking produces) and the per-group sums of x.
+      // Rows past nt are never read (their lanes read the zero row); their group sums are cleared
+      // once per tile (nobody writes them afterwards).
+      if (s0 == 0 && t0 > 0 && nt < tt)
+        for (int i = threadIdx.x; i < (tt - nt) * groups_per_slab; i += 256)
+          lds_gs[(i / (tt - nt)) * TT + nt + i % (tt - nt)] = 0.f;
+      // wave w stages token slots w, w+4, ...: the source row is wave-uniform (read from the
+      // record through the scalar cache) and every load of a row is issued before the first use
+      for (int ts = wave; ts < nt; ts += 4) {
+        const int64_t r = r0 + t0 + ts;
+        int64_t src = r;
+        if (rec_src && t0 + ts < 12) src = a.work[(size_t)blockIdx.y * 16 + 4 + t0 + ts];
+        else if (a.src_rows) src = a.src_rows[r];
+        const uint16_t *xr = a.x + src * K + s0;
+        for (int b0 = 0; b0 < sl / 8; b0 += 256) {
+          uint4 v[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int blk = b0 + j * 64 + lane;
+            v[j] = make_uint4(0, 0, 0, 0);
+            if (blk < sl / 8) v[j] = *reinterpret_cast<const uint4 *>(xr + blk * 8);
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int blk = b0 + j * 64 + lane;
+            const uint4 w = v[j];
+            float sum = ((bf16lo_to_f32(w.x) + bf16hi_to_f32(w.x)) + (bf16lo_to_f32(w.y) + bf16hi_to_f32(w.y))) +
+                        ((bf16lo_to_f32(w.z) + bf16hi_to_f32(w.z)) + (bf16lo_to_f32(w.w) + bf16hi_to_f32(w.w)));
+            sum += __shfl_xor(sum, 1, kWave);
+            sum += __shfl_xor(sum, 2, kWave);
+            sum += __shfl_xor(sum, 4, kWave);
+            if (blk < sl / 8) {
+              uint4 p = w;
+              if (BITS == 4 && !a.x_paired) {
+                p.x = (w.x & 0xffffu) | (w.z << 16);
+                p.y = (w.x >> 16) | (w.z & 0xffff0000u);
+                p.z = (w.y & 0xffffu) | (w.w << 16);
+                p.w = (w.y >> 16) | (w.w & 0xffff0000u);
+              }
+              *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = p;
+              if ((blk & 7) == 0) lds_gs[(blk >> 3) * TT + ts] = sum;
+            }
+          }
+        }
+      }
+    };
+    // after a slab has been staged: where this lane reads, and (first slab) zero accumulators
+    auto after_stage = [&](int s0) __attribute__((always_inline)) {
+      {
+        // lanes without data read the zero row
+        const int ts_l = BITS == 4 ? (c & 7) : c;
+        bool a_on = ts_l < nt;
+        if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
+        xl = lds_x + (a_on ? ts_l : tt) * xstride + kb * (CH / 4) * 2;
+        gsl = lds_gs + (BITS == 4 ? (kb >> 1) * TT + 4 * (kb & 1) : 4 * kb);
+        if (!SLABS || s0 == 0) {
+#pragma unroll
+          for (int m = 0; m < NM; ++m) tot[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+      }
+
+    };
+    // the chunks [c_first, c_last) against the slab in LDS
+    auto run_chunks = [&](int c_first, int c_last) __attribute__((always_inline)) {
+      MI_STAMP(4);
+      // D chunks in flight: slot d is refilled as soon as its chunk has been consumed.
+      if constexpr (PRECISE) {
+        int base = c_first;
+        for (; base + D <= c_last; base += D) {
+#pragma unroll
+          for (int d = 0; d < D; ++d) {
+            const int ch = base + d;
+            compute(ch, ring[d]);
+            issue(ch + D < nchunks ? ch + D : nchunks - 1, ring[d]);  // past the end: repeats of the last chunk
+          }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d)  // fewer than D chunks left (the end of the wave's range): they sit in their slots
+          if (base + d < c_last) compute(base + d, ring[d]);
+      } else {
+        for (int base = c_first; base < c_last; base += D) {
+#pragma unroll
+          for (int d = 0; d < D; ++d) {
+            const int ch = base + d;
+            if (ch < c_last) {
+              compute(ch, ring[d]);
+              if (ch + D < ch1) issue(ch + D, ring[d]);  // refill the slot just consumed
+            }
+          }
+        }
+      }
+    };
+    auto reprime = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int d = 0; d < D; ++d) {
-        const int ch = base + d;
-        if (ch < ch1) {
-          compute(ch, ring[d]);
-          if (ch + D < ch1) issue(ch + D, ring[d]);  // refill the slot just consumed
-        }
+        if constexpr (PRECISE) issue(ch0 + d < nchunks ? ch0 + d : nchunks - 1, ring[d]);
+        else if (ch0 + d < ch1) issue(ch0 + d, ring[d]);
+      }
+    };
+    if constexpr (!SLABS) {
+      __syncthreads();  // zero fill done / every wave is done reading the previous tile
+      if (t0 > 0) reprime();
+      stage_rows(0, K);
+      MI_STAMP(2);
+      __syncthreads();
+      MI_STAMP(3);
+      after_stage(0);
+      run_chunks(ch0, ch1);
+    } else {
+      for (int s0 = 0; s0 < K; s0 += sk) {
+        const int sl = K - s0 < sk ? K - s0 : sk;  // K values of this slab
+        __syncthreads();  // every wave is done reading the previous slab or tile
+        slab_ch0 = s0 / CH;
+        if (s0 == 0 && t0 > 0) reprime();
+        stage_rows(s0, sl);
+        __syncthreads();
+        after_stage(s0);
+        // this wave's chunks inside the slab.  Slabs and (when K is split over the waves) the waves'
+        // ranges start at multiples of D chunks, so a chunk keeps the ring slot (ch - ch0) % D.
+        const int slab_ch1 = (s0 + sl) / CH;
+        run_chunks(ch0 > slab_ch0 ? ch0 : slab_ch0, ch1 < slab_ch1 ? ch1 : slab_ch1);
       }
     }
 
@@ -413,28 +482,78 @@ void qmm_small_kernel(GroupedArgs a, int tt) {
   }
 }
 
+// A kernel gets 64 KB of dynamic LDS without asking.  More is asked for on every such launch (the
+// attribute belongs to the device's copy of the kernel; the call is a table update on the host).
+// An error is left for hipGetLastError() of the caller.
+static bool allow_lds(const void *fn, size_t lds) {
+  if (lds <= 64 * 1024) return true;
+  return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess;
+}
+
 template <int BITS, bool GLU>
 static void launch_small(const GroupedArgs &a, hipStream_t st) {
   constexpr int TT = BITS == 4 ? 8 : 16;  // token slots of one MFMA tile
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
-  int tt = TT;
+  int want = TT;
   // short segments on average: stage fewer rows, the LDS saved buys a fourth block per CU
-  if (a.total_rows <= 3 * (int64_t)a.max_active && tt > 4) tt = 4;
-  if (a.max_rows_per_expert < tt) tt = (int)a.max_rows_per_expert;
-  const size_t lds_budget = 60 * 1024;
-  while (tt > 1 && small_lds_bytes(a.K, tt, TT, GLU ? 4 : 2) > lds_budget) --tt;
-  const size_t lds = small_lds_bytes(a.K, tt, TT, GLU ? 4 : 2);
+  if (a.total_rows <= 3 * (int64_t)a.max_active && want > 4) want = 4;
+  if (a.max_rows_per_expert < want) want = (int)a.max_rows_per_expert;
+  // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is
+  // traded for occupancy only down to about twice the average segment; below that the tile keeps
+  // its rows even if a CU then holds one block.  Rows longer than 4096 values are staged in slabs
+  // of 4096 (2048 if that is what it takes to keep the rows: the scale/bias tiles of a long row
+  // are large too); the weight stream runs on across the slabs.
+  const size_t lds_soft = 60 * 1024, lds_hard = 150 * 1024;  // + up to 8 KB of static LDS (K-split reduction) under the 160 KB of a CU
+  const int64_t avg2 = (2 * a.total_rows + a.max_active - 1) / a.max_active;
+  const int need = (int)(avg2 < 1 ? 1 : (avg2 < want ? avg2 : want));
+  auto fit = [&](int slab) {
+    int t = want;
+    while (t > need && small_lds_bytes(a.K, slab, t, TT, GLU ? 4 : 2) > lds_soft) --t;
+    while (t > 1 && small_lds_bytes(a.K, slab, t, TT, GLU ? 4 : 2) > lds_hard) --t;
+    return t;
+  };
+  int sk = a.K;  // the whole row if the tokens wanted fit beside it
+  int tt = fit(sk);
+  if (tt < need && a.K > 4096) {
+    sk = 4096;
+    tt = fit(sk);
+    if (tt < need && fit(2048) > tt) {
+      sk = 2048;
+      tt = fit(sk);
+    }
+  }
+  const bool slabs = sk < a.K;
+  const size_t lds = small_lds_bytes(a.K, sk, tt, TT, GLU ? 4 : 2);
   // split K over the 4 waves of a block when there are too few row tiles to fill the chip
   const int64_t tiles = (int64_t)(a.N / 16) * a.max_active;
   const int chunks = a.K / (BITS == 4 ? 128 : 64);
   int kw = 1;  // measured on the 128-expert layer: 2 pays below ~2000 row tiles, 4 only when nearly empty
   if (tiles < 256 && chunks >= 8) kw = 4;
   else if (tiles < 2048 && chunks >= 4) kw = 2;
+  // with slabs a chunk's ring slot must not depend on the slab: the waves' K ranges have to start
+  // at multiples of the ring depth
+  if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % MI_MOE_RING != 0) kw = 1;
   const int nw = 4 / kw;
   dim3 grid((unsigned)((a.N + 16 * nw - 1) / (16 * nw)), (unsigned)a.max_active);
-  if (kw == 4) qmm_small_kernel<BITS, GLU, 4><<<grid, 256, lds, st>>>(a, tt);
-  else if (kw == 2) qmm_small_kernel<BITS, GLU, 2><<<grid, 256, lds, st>>>(a, tt);
-  else qmm_small_kernel<BITS, GLU, 1><<<grid, 256, lds, st>>>(a, tt);
+  // blocks a CU holds: by LDS (160 KB) and by registers (4 with the gate/up kernel, 6 otherwise)
+  const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
+  const bool precise = (by_lds < (GLU ? 4 : 6) ? by_lds : (GLU ? 4 : 6)) <= MI_MOE_PRECISE_BELOW;
+#define MI_SMALL_LAUNCH(KWV, PR, SL)                                                             \
+  do {                                                                                         \
+    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL>), lds)) return; \
+    qmm_small_kernel<BITS, GLU, KWV, PR, SL><<<grid, 256, lds, st>>>(a, tt, sk);               \
+  } while (0)
+#define MI_SMALL(KWV)                                                                          \
+  do {                                                                                         \
+    if (slabs) MI_SMALL_LAUNCH(KWV, true, true); /* long rows: few blocks per CU anyway */      \
+    else if (precise) MI_SMALL_LAUNCH(KWV, true, false);                                       \
+    else MI_SMALL_LAUNCH(KWV, false, false);                                                   \
+  } while (0)
+  if (kw == 4) MI_SMALL(4);
+  else if (kw == 2) MI_SMALL(2);
+  else MI_SMALL(1);
+#undef MI_SMALL_LAUNCH
+#undef MI_SMALL
 }
 
 // the streaming kernel on its own: segments the dispatch did not list as M tiles

@@ -52,6 +52,14 @@ def test_eight_bit(orc):
     _run_case(orc, 512, 8, 2, 1024, 8, 40, 2, seed=5)
 
 
+@pytest.mark.parametrize("T,I,bits", [(1, 6144, 4), (20, 6144, 4), (20, 6144, 8), (5, 4608, 8), (70, 8192, 4)])
+def test_long_rows_are_staged_in_slabs(orc, T, I, bits):
+    # the down product's rows are I long: beyond 4096 values the streaming kernel stages them a
+    # slab at a time (whole and partial last slabs, K split over the waves at T = 1, several
+    # passes over a segment at T = 70)
+    _run_case(orc, 256, 8, 2, I, bits, T, 0, seed=60 + T)
+
+
 def test_long_segments_and_imbalance(orc):
     # segments longer than one token tile, strongly skewed routing
     _run_case(orc, 256, 16, 4, 256, 4, 300, 0, seed=6, zipf_s=1.3)

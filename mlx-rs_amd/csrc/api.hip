@@ -107,8 +107,9 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   // (the tiled kernel reads scales in 8-byte pieces: rows of scales must be 4-byte aligned, i.e.
   // an even number of groups per row; other shapes stay on the streaming kernel)
   const bool tiled_ok = (c.hidden / 64) % 2 == 0 && (c.intermediate / 64) % 2 == 0;
-  f.tiled = T >= kTiledMinTokens && tiled_ok;
-  f.max_mtiles = f.tiled ? (int)(P / kBigTileM + (P / kTileMinRows < c.n_experts ? P / kTileMinRows : c.n_experts)) : 0;
+  f.tiled = tiled_ok && tiled_batch(P, c.n_experts, c.bits);
+  const int tmr = tile_min_rows(c.bits);
+  f.max_mtiles = f.tiled ? (int)(P / kBigTileM + (P / tmr < c.n_experts ? P / tmr : c.n_experts)) : 0;
   f.mtiles = cv.take<uint32_t>(tile_list_words(f.max_mtiles, c.n_experts));
   f.perm = cv.take<uint32_t>((size_t)P);
   f.inv_perm = cv.take<uint32_t>((size_t)P);
@@ -241,7 +242,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
                                c.n_experts, c.top_k,
                                c.score_mode, f.logits, f.topk_idx, f.topk_w, h->counters, f.counts, f.offsets,
                                f.perm, f.inv_perm, f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles,
-                               kTileMinRows, st));
+                               tile_min_rows(c.bits), st));
     MI_STAGE_DONE();
     MI_STAGE_DONE();
     MI_STAGE_DONE();
@@ -251,7 +252,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
     MI_STAGE_DONE();
     MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
-                           f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles, kTileMinRows,
+                           f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles, tile_min_rows(c.bits),
                            f.disp_scratch, st));
     MI_STAGE_DONE();
   }
@@ -523,7 +524,7 @@ static size_t qmm_dense_bytes(int64_t M, int32_t K, int32_t bits, size_t *mt_wor
   const size_t ntiles = (size_t)((M + kBigTileM - 1) / kBigTileM);
   *mt_words = tile_list_words((int)ntiles, 1);
   size_t b = 256 + 64 + *mt_words * 4 + 256;
-  if (bits == 4 && M >= kTileMinRows) b += (size_t)M * K * 2 + 256;
+  if (bits == 4 && M >= tiled_avg_rows(bits)) b += (size_t)M * K * 2 + 256;
   return b;
 }
 
@@ -565,11 +566,12 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
   Carver cv(workspace);
   uint32_t *work = cv.take<uint32_t>(16);
   uint32_t *mtiles = cv.take<uint32_t>(mt_words);
-  const bool big = M >= kTileMinRows && (K / 64) % 2 == 0;
+  // one segment of M rows: the tiled kernel from the batch threshold on (fewer rows: streaming passes)
+  const bool big = M >= tiled_avg_rows(bits) && (K / 64) % 2 == 0;
   uint16_t *xperm = (bits == 4 && big) ? cv.take<uint16_t>((size_t)M * K) : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int cap256 = (int)((M + kBigTileM - 1) / kBigTileM);
-  MI_HIP(launch_dense_records(M, big ? kTileMinRows : 0, work, mtiles, cap256, st));
+  MI_HIP(launch_dense_records(M, big ? tiled_avg_rows(bits) : 0, work, mtiles, cap256, st));
   if (xperm) MI_HIP(launch_pair_rows(x, M, K, xperm, st));
   GroupedArgs a{};
   a.x = x;

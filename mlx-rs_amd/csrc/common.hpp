@@ -7,8 +7,21 @@
 namespace mi_moe {
 
 constexpr int kWave = 64;
-constexpr int kTiledMinTokens = 192; // batches from this size on cut their longer segments into M tiles
-constexpr int kTileMinRows = 9;      // ... the segments of at least this many rows (up to 8: one pass of the streaming kernel)
+// Which rows go to the tiled MFMA kernel.  A batch uses it from an average of tiled_avg_rows(bits)
+// rows per expert on (below that nearly every segment is cheaper on the streaming kernel, and the
+// tiled launches would run empty); in such a batch the segments of at least tile_min_rows(bits) rows
+// are cut into M tiles, shorter ones stream.  Measured crossovers: see the design notes.
+#ifndef MI_TMR4
+#define MI_TMR4 9
+#define MI_TMR8 9
+#define MI_TAVG4 20
+#define MI_TAVG8 12
+#endif
+__host__ __device__ constexpr int tile_min_rows(int bits) { return bits == 4 ? MI_TMR4 : MI_TMR8; }
+__host__ __device__ constexpr int tiled_avg_rows(int bits) { return bits == 4 ? MI_TAVG4 : MI_TAVG8; }
+inline bool tiled_batch(int64_t pairs, int n_experts, int bits) {
+  return pairs >= (int64_t)tiled_avg_rows(bits) * n_experts;
+}
 constexpr int kBigTileM = 256;       // rows of the largest M tile
 constexpr int kFusedRouterMaxTokens = 64;  // up to here router + dispatch run as one launch
 
@@ -120,7 +133,7 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 
 // ---------------------------------------------------------------- M-tile lists
 // Three lists, for tiles of 256, 128 and 64 rows, back to back in one buffer: a segment of at least
-// kTileMinRows rows is cut into 256-row tiles; what is left goes to the smallest class that holds
+// tile_min_rows(bits) rows is cut into 256-row tiles; what is left goes to the smallest class that holds
 // it.  List layout: word 0 = number of tiles, tile i at words 4 + 4 i = {expert, first sorted row,
 // rows, 0}.  Capacities: cap256 for the first list, n_experts for the other two (a segment leaves
 // at most one remainder).

@@ -26,9 +26,10 @@
  *    a time (MLX itself is not thread safe, .github/workflows/validate.yml:46), and
  *    forwards through one handle must not overlap on the GPU (use one stream per handle):
  *    a handle owns 260 bytes of device memory (arrival counters of the decode router
- *    kernel) and three streams with four events (default priority; a forward of 192 tokens
- *    or more forks its independent kernel chains onto them from `stream` and joins them
- *    back before it returns, which is also what a graph capture of `stream` records), all
+ *    kernel) and three streams with four events (default priority; a prefill-sized forward,
+ *    from an average of 20 rows per expert on (12 with 8-bit weights), forks its independent
+ *    kernel chains onto them from `stream` and joins them back before it returns, which is
+ *    also what a graph capture of `stream` records), all
  *    created by mi_moe_create on the current device and released by mi_moe_destroy.  No
  *    other entry point allocates device memory or creates streams.
  *

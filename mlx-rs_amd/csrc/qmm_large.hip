@@ -33,6 +33,11 @@ constexpr int BK = 32;         // K step (two steps per quantisation group)
 constexpr int BR = 256;        // weight rows per block (GLU: 128 gate + 128 up)
 constexpr int NTHREADS = 512;  // 8 waves: 2 (token halves) x 4 (weight-row quarters)
 constexpr int DEPTH = 4;       // register stages: three K steps of global loads in flight
+#ifndef MI_SPREAD_BELOW
+#define MI_SPREAD_BELOW 64
+#endif
+constexpr int kSpreadBelow = MI_SPREAD_BELOW;  // M tiles in a list below which its N tiles are dealt over the XCDs
+static_assert(kSpreadBelow >= 1, "the launcher sizes the grid for kSpreadBelow - 1 M tiles");
 
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
@@ -69,20 +74,31 @@ constexpr size_t large_lds_bytes(int bm) { return (size_t)2 * (bm + BR) * LDR * 
 // bound by that dequantisation, which is still far cheaper than streaming the weights once per
 // 8 tokens.
 template <int BITS, bool GLU, int MT>
-__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT == 4 ? 2 : 4))) void qmm_large_kernel(GroupedArgs a, const uint32_t *__restrict__ tiles, int n_ntiles, int cap) {
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT == 4 ? 2 : 4))) void qmm_large_kernel(GroupedArgs a, const uint32_t *__restrict__ tiles, int n_ntiles, int cap, int chunk) {
   constexpr int NI = GLU ? 128 : 256;  // distinct output columns per block
   constexpr int BM = 64 * MT;          // token rows per block
   constexpr int NA = MT >= 2 ? MT / 2 : 1;  // 16-byte activation loads per thread and step
 
-  // block -> (M tile, N tile): blocks of one M tile share the gathered token rows, so they
-  // are given consecutive ids on ONE XCD (ids are dealt round-robin over the 8 XCDs)
-  const uint32_t n_mtiles = tiles[0];
+  // block -> (M tile, N tile).  Block ids are dealt round-robin over the 8 XCDs, each with its own
+  // L2.  Many M tiles: the blocks of one M tile share its gathered token rows, so they get
+  // consecutive ids on ONE XCD.  Few M tiles (a small batch, or few experts with wide matrices):
+  // whole tiles per XCD would leave XCDs idle (one M tile of a 14336-wide GLU is 112 blocks, all on
+  // one XCD's 32 CUs), so the N tiles of an M tile are dealt over the XCDs in chunks of `chunk`.
+  // Both candidate records are fetched along with the count (indices clamped to the list's capacity).
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-  const int nt = j % n_ntiles;
-  const uint32_t mt_id = (uint32_t)(j / n_ntiles) * 8u + xcd;
-  // the record is fetched along with the count (index clamped to the list's capacity)
-  const uint4 rec = reinterpret_cast<const uint4 *>(tiles)[1 + (mt_id < (uint32_t)cap ? mt_id : (uint32_t)cap - 1u)];
-  if (mt_id >= n_mtiles) return;
+  const int n_chunks = (n_ntiles + chunk - 1) / chunk;
+  const uint32_t whole_id = (uint32_t)(j / n_ntiles) * 8u + xcd;
+  const uint32_t unit = (uint32_t)(j / chunk) * 8u + xcd;
+  const uint32_t spread_id = unit / (uint32_t)n_chunks;
+  const uint4 *const recs = reinterpret_cast<const uint4 *>(tiles) + 1;
+  const uint4 rec_whole = recs[whole_id < (uint32_t)cap ? whole_id : (uint32_t)cap - 1u];
+  const uint4 rec_spread = recs[spread_id < (uint32_t)cap ? spread_id : (uint32_t)cap - 1u];
+  const uint32_t n_mtiles = tiles[0];
+  const bool spread = n_mtiles < (uint32_t)kSpreadBelow;
+  const uint32_t mt_id = spread ? spread_id : whole_id;
+  const int nt = spread ? (int)(unit % (uint32_t)n_chunks) * chunk + j % chunk : j % n_ntiles;
+  const uint4 rec = spread ? rec_spread : rec_whole;
+  if (mt_id >= n_mtiles || nt >= n_ntiles) return;
   const int e = (int)rec.x;
   const int64_t row0 = rec.y;
   const int rows = (int)rec.z;
@@ -386,7 +402,13 @@ template <int BITS, bool GLU, int MT>
 static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int cap, hipStream_t st) {
   const int ni = GLU ? 128 : 256;
   const int n_ntiles = (a.N + ni - 1) / ni;
-  const unsigned grid = (unsigned)((cap + 7) / 8) * 8u * (unsigned)n_ntiles;
+  // ids for either dealing of the tiles (see the kernel): whole M tiles per XCD, or chunks of an
+  // M tile's N tiles when the list holds fewer than kSpreadBelow M tiles
+  const int chunk = (n_ntiles + 7) / 8, n_chunks = (n_ntiles + chunk - 1) / chunk;
+  const unsigned whole = (unsigned)((cap + 7) / 8) * 8u * (unsigned)n_ntiles;
+  const unsigned few = (unsigned)(cap < kSpreadBelow - 1 ? cap : kSpreadBelow - 1);
+  const unsigned spread = (few * (unsigned)n_chunks + 7u) / 8u * 8u * (unsigned)chunk;
+  const unsigned grid = whole > spread ? whole : spread;
   constexpr size_t lds = large_lds_bytes(64 * MT);
   // more LDS per block than a kernel gets without asking: asked for once per device (the attribute
   // belongs to the device's copy of the kernel); two threads asking at once is harmless
@@ -401,7 +423,7 @@ static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int ca
       return e;
     if (dev >= 0 && dev < kMaxDevices) raised[dev].store(true, std::memory_order_release);
   }
-  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles, cap);
+  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles, cap, chunk);
   return hipGetLastError();
 }
 

@@ -86,7 +86,9 @@ struct ForwardWs {
   uint16_t *topk_w;
   uint32_t *counts, *offsets, *work, *mtiles, *perm, *inv_perm, *src_of;
   int max_mtiles;
-  bool tiled;
+  bool tiled;  // tile lists are built
+  bool heavy;  // most rows are tiled: see heavy_batch()
+  int tmr;     // segments of at least this many rows are tiled
   void *disp_scratch;
   uint16_t *hh, *y, *xperm, *xnorm;
   size_t bytes;
@@ -108,7 +110,8 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   // an even number of groups per row; other shapes stay on the streaming kernel)
   const bool tiled_ok = (c.hidden / 64) % 2 == 0 && (c.intermediate / 64) % 2 == 0;
   f.tiled = tiled_ok && tiled_batch(P, c.n_experts, c.bits);
-  const int tmr = tile_min_rows(c.bits);
+  f.heavy = f.tiled && heavy_batch(P, c.n_experts, c.bits);
+  const int tmr = f.tmr = tile_min_rows(c.bits, f.heavy);
   f.max_mtiles = f.tiled ? (int)(P / kBigTileM + (P / tmr < c.n_experts ? P / tmr : c.n_experts)) : 0;
   f.mtiles = cv.take<uint32_t>(tile_list_words(f.max_mtiles, c.n_experts));
   f.perm = cv.take<uint32_t>((size_t)P);
@@ -133,7 +136,7 @@ struct mi_moe_s {
   // (gate/up then down over the same rows); three of the four run on these streams, forked from
   // and joined back into the caller's stream by events
   hipStream_t side[3] = {nullptr, nullptr, nullptr};
-  hipEvent_t fork = nullptr, join[3] = {nullptr, nullptr, nullptr};
+  hipEvent_t fork = nullptr, paired = nullptr, join[3] = {nullptr, nullptr, nullptr};
 };
 
 void destroy_handle(mi_moe_s *h) {
@@ -144,6 +147,7 @@ void destroy_handle(mi_moe_s *h) {
     if (h->join[i]) (void)hipEventDestroy(h->join[i]);
   }
   if (h->fork) (void)hipEventDestroy(h->fork);
+  if (h->paired) (void)hipEventDestroy(h->paired);
   delete h;
 }
 
@@ -183,6 +187,7 @@ int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_mo
     if (e == hipSuccess) e = hipEventCreateWithFlags(&h->join[i], hipEventDisableTiming);
   }
   if (e == hipSuccess) e = hipEventCreateWithFlags(&h->fork, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&h->paired, hipEventDisableTiming);
   if (e != hipSuccess) {
     destroy_handle(h);
     return fail("create: device memory, streams and events of the handle: %s", hipGetErrorString(e));
@@ -242,7 +247,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
                                c.n_experts, c.top_k,
                                c.score_mode, f.logits, f.topk_idx, f.topk_w, h->counters, f.counts, f.offsets,
                                f.perm, f.inv_perm, f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles,
-                               tile_min_rows(c.bits), st));
+                               f.tmr, st));
     MI_STAGE_DONE();
     MI_STAGE_DONE();
     MI_STAGE_DONE();
@@ -252,7 +257,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
     MI_STAGE_DONE();
     MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
-                           f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles, tile_min_rows(c.bits),
+                           f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles, f.tmr,
                            f.disp_scratch, st));
     MI_STAGE_DONE();
   }
@@ -269,7 +274,9 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   // 4-bit: the tiled kernel reads activations with paired 8-blocks; h is produced that way,
   // x is copied once per forward (prefill-sized T only)
   const bool paired = c.bits == 4;
-  if (f.tiled && paired) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
+  // light batches start their streamed segments first and pair the rows beside them (below)
+  const bool streamed_first = f.tiled && !f.heavy && !ev;
+  if (f.tiled && paired && !streamed_first) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
   // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
   a.x = x;
   a.x_perm = paired ? (f.tiled ? f.xperm : nullptr) : x;
@@ -300,18 +307,35 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   if (large_qmm_applies(a) && !ev) {
     // Four chains that share no rows: the three tile classes and the streamed segments, each
     // gate/up then down.  The short classes leave most of the chip idle when they run alone
-    // (a few dozen workgroups of 64 K steps each); side by side they fill it.  The longest chain
-    // stays on the caller's stream.
+    // (a few dozen workgroups of 64 K steps each); side by side they fill it.  The chain that is
+    // expected to be the longest stays on the caller's stream and is launched first: the 256-row
+    // class of a heavy batch, the streamed segments of a light one (whose tile lists are empty
+    // unless the routing is uneven; the copy of x with paired rows, which only the tiles read,
+    // then runs on a side stream as well).
     MI_HIP(hipEventRecord(h->fork, st));
     for (int i = 0; i < 3; ++i) MI_HIP(hipStreamWaitEvent(h->side[i], h->fork, 0));
-    for (int chain = 0; chain < 4; ++chain) {
-      hipStream_t s = chain == 0 ? st : h->side[chain - 1];
-      if (chain < 3) {
-        MI_HIP(launch_large_qmm_class(a, true, chain, s));
-        MI_HIP(launch_large_qmm_class(d, false, chain, s));
-      } else {
-        MI_HIP(launch_small_qmm(a, true, s));
-        MI_HIP(launch_small_qmm(d, false, s));
+    if (streamed_first) {
+      MI_HIP(launch_small_qmm(a, true, st));
+      MI_HIP(launch_small_qmm(d, false, st));
+      if (paired) {
+        MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, h->side[0]));
+        MI_HIP(hipEventRecord(h->paired, h->side[0]));
+        for (int i = 1; i < 3; ++i) MI_HIP(hipStreamWaitEvent(h->side[i], h->paired, 0));
+      }
+      for (int cls = 0; cls < 3; ++cls) {
+        MI_HIP(launch_large_qmm_class(a, true, cls, h->side[cls]));
+        MI_HIP(launch_large_qmm_class(d, false, cls, h->side[cls]));
+      }
+    } else {
+      for (int chain = 0; chain < 4; ++chain) {
+        hipStream_t s = chain == 0 ? st : h->side[chain - 1];
+        if (chain < 3) {
+          MI_HIP(launch_large_qmm_class(a, true, chain, s));
+          MI_HIP(launch_large_qmm_class(d, false, chain, s));
+        } else {
+          MI_HIP(launch_small_qmm(a, true, s));
+          MI_HIP(launch_small_qmm(d, false, s));
+        }
       }
     }
     for (int i = 0; i < 3; ++i) {

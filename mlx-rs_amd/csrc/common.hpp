@@ -7,20 +7,36 @@
 namespace mi_moe {
 
 constexpr int kWave = 64;
-// Which rows go to the tiled MFMA kernel.  A batch uses it from an average of tiled_avg_rows(bits)
-// rows per expert on (below that nearly every segment is cheaper on the streaming kernel, and the
-// tiled launches would run empty); in such a batch the segments of at least tile_min_rows(bits) rows
-// are cut into M tiles, shorter ones stream.  Measured crossovers: see the design notes.
+// Which rows go to the tiled MFMA kernel.  A batch with an average of at least tiled_avg_rows(bits)
+// rows per expert is "heavy": most segments are worth a tile, those of tile_min_rows(bits, true) rows
+// or more (beyond one pass of the streaming kernel) are cut into M tiles, shorter ones stream.
+// From light_avg_rows(bits) on a batch is "light": with even routing nearly every segment is cheaper
+// on the streaming kernel, but a popular expert's segment is many passes long there (250 rows of a
+// 256-token batch: 30 passes over that expert's weights), so segments of tile_min_rows(bits, false)
+// rows or more (beyond two passes) are tiled.  Below light_avg_rows everything streams and the tile
+// lists are not built.  Measured crossovers: see the design notes.
 #ifndef MI_TMR4
 #define MI_TMR4 9
 #define MI_TMR8 9
 #define MI_TAVG4 20
 #define MI_TAVG8 12
 #endif
-__host__ __device__ constexpr int tile_min_rows(int bits) { return bits == 4 ? MI_TMR4 : MI_TMR8; }
+#ifndef MI_TLIGHT4
+#define MI_TLIGHT4 6
+#define MI_TLIGHT8 12
+#define MI_TMRL4 17
+#define MI_TMRL8 9
+#endif
+__host__ __device__ constexpr int tile_min_rows(int bits, bool heavy) {
+  return bits == 4 ? (heavy ? MI_TMR4 : MI_TMRL4) : (heavy ? MI_TMR8 : MI_TMRL8);
+}
 __host__ __device__ constexpr int tiled_avg_rows(int bits) { return bits == 4 ? MI_TAVG4 : MI_TAVG8; }
-inline bool tiled_batch(int64_t pairs, int n_experts, int bits) {
+__host__ __device__ constexpr int light_avg_rows(int bits) { return bits == 4 ? MI_TLIGHT4 : MI_TLIGHT8; }
+inline bool heavy_batch(int64_t pairs, int n_experts, int bits) {
   return pairs >= (int64_t)tiled_avg_rows(bits) * n_experts;
+}
+inline bool tiled_batch(int64_t pairs, int n_experts, int bits) {
+  return pairs >= (int64_t)light_avg_rows(bits) * n_experts || heavy_batch(pairs, n_experts, bits);
 }
 constexpr int kBigTileM = 256;       // rows of the largest M tile
 constexpr int kFusedRouterMaxTokens = 64;  // up to here router + dispatch run as one launch
@@ -133,7 +149,7 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 
 // ---------------------------------------------------------------- M-tile lists
 // Three lists, for tiles of 256, 128 and 64 rows, back to back in one buffer: a segment of at least
-// tile_min_rows(bits) rows is cut into 256-row tiles; what is left goes to the smallest class that holds
+// tile_min_rows(bits, heavy) rows is cut into 256-row tiles; what is left goes to the smallest class that holds
 // it.  List layout: word 0 = number of tiles, tile i at words 4 + 4 i = {expert, first sorted row,
 // rows, 0}.  Capacities: cap256 for the first list, n_experts for the other two (a segment leaves
 // at most one remainder).

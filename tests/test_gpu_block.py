@@ -116,6 +116,14 @@ def test_tile_classes(orc, T, E, k, bits, zipf):
     _run_case(orc, 256, E, k, 384, bits, T, 0, seed=31 + T, zipf_s=zipf)
 
 
+@pytest.mark.parametrize("T,E,k,zipf", [(100, 16, 2, 1.5), (40, 16, 4, 1.2), (150, 32, 4, 1.0), (150, 32, 4, None)])
+def test_light_batches_tile_only_long_segments(orc, T, E, k, zipf):
+    # 6 to 20 rows per expert on average (4-bit): the streamed segments lead on the caller's stream,
+    # segments of 17 rows and more (uneven routing) are tiled on the side streams; 40 tokens: the
+    # one-launch router builds the tile lists
+    _run_case(orc, 256, E, k, 384, 4, T, 0, seed=57 + T, zipf_s=zipf)
+
+
 @pytest.mark.parametrize("T,H,E,k,I,bits,mode,zipf", [(1, 256, 8, 2, 512, 4, 0, None), (32, 2048, 128, 8, 768, 4, 0, None),
                                                       (300, 256, 16, 4, 256, 8, 2, 1.0)])
 def test_norm_and_residual_around_the_block(orc, T, H, E, k, I, bits, mode, zipf):
@@ -150,11 +158,12 @@ def test_norm_and_residual_around_the_block(orc, T, H, E, k, I, bits, mode, zipf
         blk.forward_residual(xd, nwd, 1e-6, out=xd)
 
 
-@pytest.mark.parametrize("T", [4, 300])
+@pytest.mark.parametrize("T", [4, 70, 300])
 def test_graph_replays_equal_eager(orc, T):
     """A forward captured into a HIP graph (decode: the one-launch router with its self-resetting
-    arrival counters; prefill: the tiled kernels) gives the eager result on every replay, with
-    eager forwards of other sizes and synchronisations in between."""
+    arrival counters; 70 tokens: streamed segments first, tiles beside them; prefill: the tiled
+    kernels) gives the eager result on every replay, with eager forwards of other sizes and
+    synchronisations in between."""
     import mlx_rs_amd as m
     H, E, k, I = 256, 16, 4, 256
     W = host_layer(orc, H, E, k, I, 4, seed=77)

@@ -271,6 +271,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   a.bits = c.bits;
   a.total_rows = P;
   a.max_rows_per_expert = T;  // a token picks an expert at most once
+  a.max_streamed_rows = f.tiled ? f.tmr - 1 : 0;
   // 4-bit: the tiled kernel reads activations with paired 8-blocks; h is produced that way,
   // x is copied once per forward (prefill-sized T only)
   const bool paired = c.bits == 4;

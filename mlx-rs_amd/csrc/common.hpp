@@ -198,6 +198,7 @@ struct GroupedArgs {
   int N, K, bits;
   int64_t total_rows;          // host upper bound on rows (for tile selection)
   int64_t max_rows_per_expert; // host upper bound on the longest segment
+  int64_t max_streamed_rows;   // host upper bound on the longest segment that is not tiled (0: no bound known)
 };
 
 hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,

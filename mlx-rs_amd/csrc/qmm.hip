@@ -81,6 +81,12 @@ extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
 #ifndef MI_MOE_RING
 #define MI_MOE_RING 4
 #endif
+#ifndef MI_MOE_TG2_AVG
+#define MI_MOE_TG2_AVG 5   // rows per active expert from which the 4-bit kernel takes two token groups per pass
+#endif
+#ifndef MI_MOE_TG2_SLAB
+#define MI_MOE_TG2_SLAB 1024
+#endif
 #ifndef MI_MOE_PRECISE_BELOW
 #define MI_MOE_PRECISE_BELOW 2  // blocks per CU up to which the ring takes the unconditional form
 #endif
@@ -120,9 +126,14 @@ __host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int 
 // room for two blocks per CU only (K = 4096: 8 KB of LDS per staged token).
 // SLABS: the activation rows are staged sk K values at a time (rows too long for LDS); without it
 // sk = K and the slab loop below is a single pass the compiler folds away.
-template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS>
+// TG: token groups per pass.  A 4-bit MFMA tile holds 8 tokens (its other 8 A rows carry the same
+// tokens for the chunk's second quantisation group); with TG = 2 a chunk of weights is multiplied
+// with two such tiles, tokens 0-7 and 8-15 of the pass, before its ring slot is refilled: segments
+// of 9 to 16 rows then take one pass over the expert's weights instead of two.
+template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8)))
 void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
+  static_assert(TG == 1 || (TG == 2 && BITS == 4 && KW == 1), "two token groups: 4-bit, K not split over waves");
   constexpr int NW = 4 / KW;                    // row tiles per block
   constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one 16-byte load per lane)
   constexpr int XV = BITS == 4 ? 4 : 2;         // 16-byte pieces of activations per lane per chunk
@@ -141,6 +152,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   MI_STAMP(6);
   const bool rec_src = a.src_in_work && rec0.w != 0u;
   constexpr int TT = BITS == 4 ? 8 : 16;        // token slots of one MFMA tile
+  constexpr int TTL = TT * TG;                  // token slots of one pass
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction
   const int wk = wave % KW, wn = wave / KW;
@@ -210,8 +222,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
   extern __shared__ __align__(16) unsigned char lds[];
   unsigned char *lds_x = lds;
-  float *lds_gs = reinterpret_cast<float *>(lds + (tt + 1) * xstride);  // [groups of the slab][TT] sums of x
-  unsigned char *lds_sb = lds + (tt + 1) * xstride + groups_per_slab * TT * 4 + wave * NTEN * sbt;
+  float *lds_gs = reinterpret_cast<float *>(lds + (tt + 1) * xstride);  // [groups of the slab][TTL] sums of x
+  unsigned char *lds_sb = lds + (tt + 1) * xstride + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
 
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait)
 #pragma unroll
@@ -231,73 +243,78 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   // zero row and zero group sums (slots that carry no token stay zero for the whole launch)
   for (int i = threadIdx.x; i < xstride / 16; i += 256)
     *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
-  for (int i = threadIdx.x; i < groups_per_slab * TT / 4; i += 256)
+  for (int i = threadIdx.x; i < groups_per_slab * TTL / 4; i += 256)
     *reinterpret_cast<uint4 *>(lds_gs + i * 4) = make_uint4(0, 0, 0, 0);
 
   for (int t0 = 0; t0 < cnt; t0 += tt) {
     const int nt = cnt - t0 < tt ? cnt - t0 : tt;  // tokens of this tile
 
     // set after a slab has been staged (kept out of the staging's way: they cost registers there)
-    const unsigned char *xl;  // activation row of this lane (A operand)
-    const float *gsl;         // group sums of x for this lane's 4 D rows (token slots), first group of the slab
-    f32x4_t tot[NM];
+    const unsigned char *xl[TG];  // activation row of this lane (A operand), per token group
+    const float *gsl;             // group sums of x for this lane's 4 D rows (token slots), first group of the slab
+    f32x4_t tot[TG][NM];
     int slab_ch0 = 0;  // first chunk of the slab that is in LDS
 
     // one chunk: MFMAs on raw codes, then scale and bias applied to the fp32 group sums
     auto compute = [&](int ch, const Regs &R) {
-      uint4 xv[XV];
 #pragma unroll
-      for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl + (SLABS ? ch - slab_ch0 : ch) * CH * 2 + i * 16);
-      f32x4_t acc[NM];
+      for (int g = 0; g < TG; ++g) {
+        // the groups one after the other: interleaved, both groups' activations would be live at once
+        if (TG > 1 && g > 0) __builtin_amdgcn_sched_barrier(0);
+        uint4 xv[XV];
 #pragma unroll
-      for (int m = 0; m < NM; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if constexpr (BITS == 4) {
+        for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl[g] + (SLABS ? ch - slab_ch0 : ch) * CH * 2 + i * 16);
+        f32x4_t acc[NM];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const uint32_t av[4] = {xv[s].x, xv[s].y, xv[s].z, xv[s].w};
+        for (int m = 0; m < NM; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if constexpr (BITS == 4) {
 #pragma unroll
-          for (int m = 0; m < NM; ++m) {
-            const uint32_t w = R.q[m][s];
-            uint32_t bv[4];
-            bv[0] = and_or(w, nib_mask, nib_magic);
-            bv[1] = and_or(w >> 4, nib_mask, nib_magic);
-            bv[2] = and_or(w >> 8, nib_mask, nib_magic);
-            bv[3] = and_or(w >> 12, nib_mask, nib_magic);
-            acc[m] = mfma16(av, bv, acc[m]);
+          for (int s = 0; s < 4; ++s) {
+            const uint32_t av[4] = {xv[s].x, xv[s].y, xv[s].z, xv[s].w};
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+              const uint32_t w = R.q[m][s];
+              uint32_t bv[4];
+              bv[0] = and_or(w, nib_mask, nib_magic);
+              bv[1] = and_or(w >> 4, nib_mask, nib_magic);
+              bv[2] = and_or(w >> 8, nib_mask, nib_magic);
+              bv[3] = and_or(w >> 12, nib_mask, nib_magic);
+              acc[m] = mfma16(av, bv, acc[m]);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const uint32_t av[4] = {xv[s].x, xv[s].y, xv[s].z, xv[s].w};
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+              const uint32_t wA = R.q[m][2 * s], wB = R.q[m][2 * s + 1];
+              uint32_t bv[4];
+              bv[0] = (__float_as_uint((float)(wA & 0xffu)) >> 16) |
+                      (__float_as_uint((float)((wA >> 8) & 0xffu)) & 0xffff0000u);
+              bv[1] = (__float_as_uint((float)((wA >> 16) & 0xffu)) >> 16) |
+                      (__float_as_uint((float)(wA >> 24)) & 0xffff0000u);
+              bv[2] = (__float_as_uint((float)(wB & 0xffu)) >> 16) |
+                      (__float_as_uint((float)((wB >> 8) & 0xffu)) & 0xffff0000u);
+              bv[3] = (__float_as_uint((float)((wB >> 16) & 0xffu)) >> 16) |
+                      (__float_as_uint((float)(wB >> 24)) & 0xffff0000u);
+              acc[m] = mfma16(av, bv, acc[m]);
+            }
           }
         }
-      } else {
+        // sum_c x_c (s (128 + q_c - 128) + b) = s * acc + (b - 128 s) * sum_c x_c   (8-bit: no offset)
+        const float4 xs = *reinterpret_cast<const float4 *>(gsl + (SLABS ? ch - slab_ch0 : ch) * (BITS == 4 ? 2 : 1) * TTL + TT * g);
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          const uint32_t av[4] = {xv[s].x, xv[s].y, xv[s].z, xv[s].w};
-#pragma unroll
-          for (int m = 0; m < NM; ++m) {
-            const uint32_t wA = R.q[m][2 * s], wB = R.q[m][2 * s + 1];
-            uint32_t bv[4];
-            bv[0] = (__float_as_uint((float)(wA & 0xffu)) >> 16) |
-                    (__float_as_uint((float)((wA >> 8) & 0xffu)) & 0xffff0000u);
-            bv[1] = (__float_as_uint((float)((wA >> 16) & 0xffu)) >> 16) |
-                    (__float_as_uint((float)(wA >> 24)) & 0xffff0000u);
-            bv[2] = (__float_as_uint((float)(wB & 0xffu)) >> 16) |
-                    (__float_as_uint((float)((wB >> 8) & 0xffu)) & 0xffff0000u);
-            bv[3] = (__float_as_uint((float)((wB >> 16) & 0xffu)) >> 16) |
-                    (__float_as_uint((float)(wB >> 24)) & 0xffff0000u);
-            acc[m] = mfma16(av, bv, acc[m]);
-          }
+        for (int m = 0; m < NM; ++m) {
+          const int goff = ch * (BITS == 4 ? 4 : 2);
+          const float sc = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m) * sbt + goff));
+          float bi = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m + 1) * sbt + goff));
+          if constexpr (BITS == 4) bi = __builtin_fmaf(-128.0f, sc, bi);
+          tot[g][m][0] = __builtin_fmaf(sc, acc[m][0], __builtin_fmaf(bi, xs.x, tot[g][m][0]));
+          tot[g][m][1] = __builtin_fmaf(sc, acc[m][1], __builtin_fmaf(bi, xs.y, tot[g][m][1]));
+          tot[g][m][2] = __builtin_fmaf(sc, acc[m][2], __builtin_fmaf(bi, xs.z, tot[g][m][2]));
+          tot[g][m][3] = __builtin_fmaf(sc, acc[m][3], __builtin_fmaf(bi, xs.w, tot[g][m][3]));
         }
-      }
-      // sum_c x_c (s (128 + q_c - 128) + b) = s * acc + (b - 128 s) * sum_c x_c   (8-bit: no offset)
-      const float4 xs = *reinterpret_cast<const float4 *>(gsl + (SLABS ? ch - slab_ch0 : ch) * (BITS == 4 ? 2 : 1) * TT);
-#pragma unroll
-      for (int m = 0; m < NM; ++m) {
-        const int goff = ch * (BITS == 4 ? 4 : 2);
-        const float sc = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m) * sbt + goff));
-        float bi = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m + 1) * sbt + goff));
-        if constexpr (BITS == 4) bi = __builtin_fmaf(-128.0f, sc, bi);
-        tot[m][0] = __builtin_fmaf(sc, acc[m][0], __builtin_fmaf(bi, xs.x, tot[m][0]));
-        tot[m][1] = __builtin_fmaf(sc, acc[m][1], __builtin_fmaf(bi, xs.y, tot[m][1]));
-        tot[m][2] = __builtin_fmaf(sc, acc[m][2], __builtin_fmaf(bi, xs.z, tot[m][2]));
-        tot[m][3] = __builtin_fmaf(sc, acc[m][3], __builtin_fmaf(bi, xs.w, tot[m][3]));
       }
     };
 
@@ -310,7 +327,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
       // once per tile (nobody writes them afterwards).
       if (s0 == 0 && t0 > 0 && nt < tt)
         for (int i = threadIdx.x; i < (tt - nt) * groups_per_slab; i += 256)
-          lds_gs[(i / (tt - nt)) * TT + nt + i % (tt - nt)] = 0.f;
+          lds_gs[(i / (tt - nt)) * TTL + nt + i % (tt - nt)] = 0.f;
       // wave w stages token slots w, w+4, ...: the source row is wave-uniform (read from the
       // record through the scalar cache) and every load of a row is issued before the first use
       for (int ts = wave; ts < nt; ts += 4) {
@@ -345,7 +362,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
                 p.w = (w.y >> 16) | (w.w & 0xffff0000u);
               }
               *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = p;
-              if ((blk & 7) == 0) lds_gs[(blk >> 3) * TT + ts] = sum;
+              if ((blk & 7) == 0) lds_gs[(blk >> 3) * TTL + ts] = sum;
             }
           }
         }
@@ -355,14 +372,19 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     auto after_stage = [&](int s0) __attribute__((always_inline)) {
       {
         // lanes without data read the zero row
-        const int ts_l = BITS == 4 ? (c & 7) : c;
-        bool a_on = ts_l < nt;
-        if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
-        xl = lds_x + (a_on ? ts_l : tt) * xstride + kb * (CH / 4) * 2;
-        gsl = lds_gs + (BITS == 4 ? (kb >> 1) * TT + 4 * (kb & 1) : 4 * kb);
+#pragma unroll
+        for (int g = 0; g < TG; ++g) {
+          const int ts_l = (BITS == 4 ? (c & 7) : c) + TT * g;
+          bool a_on = ts_l < nt;
+          if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
+          xl[g] = lds_x + (a_on ? ts_l : tt) * xstride + kb * (CH / 4) * 2;
+        }
+        gsl = lds_gs + (BITS == 4 ? (kb >> 1) * TTL + 4 * (kb & 1) : 4 * kb);
         if (!SLABS || s0 == 0) {
 #pragma unroll
-          for (int m = 0; m < NM; ++m) tot[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          for (int g = 0; g < TG; ++g)
+#pragma unroll
+            for (int m = 0; m < NM; ++m) tot[g][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
       }
 
@@ -432,24 +454,28 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     MI_STAMP(5);
     if constexpr (BITS == 4) {  // rows 8-15 (second group of each chunk) onto rows 0-7
 #pragma unroll
-      for (int m = 0; m < NM; ++m)
+      for (int g = 0; g < TG; ++g)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) tot[m][r] += __shfl_xor(tot[m][r], 32, kWave);
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) tot[g][m][r] += __shfl_xor(tot[g][m][r], 32, kWave);
     }
 
     // cross-wave sum over the K split, in wave order
     constexpr int LR = BITS == 4 ? 32 : 64;  // lanes that hold distinct results
-    float res[NM][4];
+    float res[TG][NM][4];
     if constexpr (KW == 1) {
 #pragma unroll
-      for (int m = 0; m < NM; ++m)
+      for (int g = 0; g < TG; ++g)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) res[m][r] = tot[m][r];
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) res[g][m][r] = tot[g][m][r];
     } else {
 #pragma unroll
       for (int m = 0; m < NM; ++m)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[wk][wn][m][r][lane] = tot[m][r];
+        for (int r = 0; r < 4; ++r) red[wk][wn][m][r][lane] = tot[0][m][r];
       __syncthreads();
 #pragma unroll
       for (int m = 0; m < NM; ++m)
@@ -458,26 +484,28 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
           float s = 0.f;
 #pragma unroll
           for (int w = 0; w < KW; ++w) s += red[w][wn][m][r][lane];
-          res[m][r] = s;
+          res[0][m][r] = s;
         }
     }
 
     // epilogue: one wave per row tile writes nt x 16 outputs
     if (wk == 0 && tile_ok && lane < LR) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int slot = BITS == 4 ? 4 * (kb & 1) + r : 4 * kb + r;
-        if (slot < nt) {
-          const int64_t rr = r0 + t0 + slot;
-          const int64_t dst = a.dst_rows ? (int64_t)a.dst_rows[rr] : rr;
-          float v;
-          if constexpr (GLU) v = silu_mul(res[0][r], res[1][r]);
-          else v = res[0][r];
-          int col = n;
-          if (a.y_paired) col = (n & ~7) | ((n & 7) < 4 ? 2 * (n & 7) : 2 * ((n & 7) - 4) + 1);
-          a.y[dst * N + col] = (uint16_t)(cvt_pk_bf16(v, 0.f) & 0xffffu);
+      for (int g = 0; g < TG; ++g)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int slot = TT * g + (BITS == 4 ? 4 * (kb & 1) + r : 4 * kb + r);
+          if (slot < nt) {
+            const int64_t rr = r0 + t0 + slot;
+            const int64_t dst = a.dst_rows ? (int64_t)a.dst_rows[rr] : rr;
+            float v;
+            if constexpr (GLU) v = silu_mul(res[g][0][r], res[g][1][r]);
+            else v = res[g][0][r];
+            int col = n;
+            if (a.y_paired) col = (n & ~7) | ((n & 7) < 4 ? 2 * (n & 7) : 2 * ((n & 7) - 4) + 1);
+            a.y[dst * N + col] = (uint16_t)(cvt_pk_bf16(v, 0.f) & 0xffffu);
+          }
         }
-      }
     }
   }
 }
@@ -493,11 +521,25 @@ static bool allow_lds(const void *fn, size_t lds) {
 template <int BITS, bool GLU>
 static void launch_small(const GroupedArgs &a, hipStream_t st) {
   constexpr int TT = BITS == 4 ? 8 : 16;  // token slots of one MFMA tile
+  // split K over the 4 waves of a block when there are too few row tiles to fill the chip
+  const int64_t tiles = (int64_t)(a.N / 16) * a.max_active;
+  const int chunks = a.K / (BITS == 4 ? 128 : 64);
+  int kw = 1;  // measured on the 128-expert layer: 2 pays below ~2000 row tiles, 4 only when nearly empty
+  if (tiles < 256 && chunks >= 8) kw = 4;
+  else if (tiles < 2048 && chunks >= 4) kw = 2;
+  // 4-bit, segments that can be longer than one MFMA tile's 8 tokens, and long enough on average
+  // for it to matter: two token groups per pass (a 9- to 16-row segment then reads its expert's
+  // weights once, not twice)
+  const int64_t longest = a.max_streamed_rows > 0 && a.max_streamed_rows < a.max_rows_per_expert
+                              ? a.max_streamed_rows : a.max_rows_per_expert;
+  const bool two_groups = BITS == 4 && kw == 1 && longest > TT &&
+                          a.total_rows >= (int64_t)MI_MOE_TG2_AVG * a.max_active;
+  const int TTL = two_groups ? 2 * TT : TT;  // token slots of one pass
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
-  int want = TT;
+  int want = TTL;
   // short segments on average: stage fewer rows, the LDS saved buys a fourth block per CU
   if (a.total_rows <= 3 * (int64_t)a.max_active && want > 4) want = 4;
-  if (a.max_rows_per_expert < want) want = (int)a.max_rows_per_expert;
+  if (longest < want) want = (int)longest;
   // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is
   // traded for occupancy only down to about twice the average segment; below that the tile keeps
   // its rows even if a CU then holds one block.  Rows longer than 4096 values are staged in slabs
@@ -508,13 +550,18 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int need = (int)(avg2 < 1 ? 1 : (avg2 < want ? avg2 : want));
   auto fit = [&](int slab) {
     int t = want;
-    while (t > need && small_lds_bytes(a.K, slab, t, TT, GLU ? 4 : 2) > lds_soft) --t;
-    while (t > 1 && small_lds_bytes(a.K, slab, t, TT, GLU ? 4 : 2) > lds_hard) --t;
+    while (t > need && small_lds_bytes(a.K, slab, t, TTL, GLU ? 4 : 2) > lds_soft) --t;
+    while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, GLU ? 4 : 2) > lds_hard) --t;
     return t;
   };
   int sk = a.K;  // the whole row if the tokens wanted fit beside it
   int tt = fit(sk);
-  if (tt < need && a.K > 4096) {
+  if (two_groups && MI_MOE_TG2_SLAB > 0 && a.K > MI_MOE_TG2_SLAB && a.K % MI_MOE_TG2_SLAB == 0 &&
+      small_lds_bytes(a.K, sk, tt, TTL, GLU ? 4 : 2) > lds_soft) {
+    // sixteen whole rows leave room for one block per CU: stage them in slabs instead
+    sk = MI_MOE_TG2_SLAB;
+    tt = fit(sk);
+  } else if (tt < need && a.K > 4096) {
     sk = 4096;
     tt = fit(sk);
     if (tt < need && fit(2048) > tt) {
@@ -523,13 +570,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
     }
   }
   const bool slabs = sk < a.K;
-  const size_t lds = small_lds_bytes(a.K, sk, tt, TT, GLU ? 4 : 2);
-  // split K over the 4 waves of a block when there are too few row tiles to fill the chip
-  const int64_t tiles = (int64_t)(a.N / 16) * a.max_active;
-  const int chunks = a.K / (BITS == 4 ? 128 : 64);
-  int kw = 1;  // measured on the 128-expert layer: 2 pays below ~2000 row tiles, 4 only when nearly empty
-  if (tiles < 256 && chunks >= 8) kw = 4;
-  else if (tiles < 2048 && chunks >= 4) kw = 2;
+  const size_t lds = small_lds_bytes(a.K, sk, tt, TTL, GLU ? 4 : 2);
   // with slabs a chunk's ring slot must not depend on the slab: the waves' K ranges have to start
   // at multiples of the ring depth
   if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % MI_MOE_RING != 0) kw = 1;
@@ -538,20 +579,26 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // blocks a CU holds: by LDS (160 KB) and by registers (4 with the gate/up kernel, 6 otherwise)
   const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
   const bool precise = (by_lds < (GLU ? 4 : 6) ? by_lds : (GLU ? 4 : 6)) <= MI_MOE_PRECISE_BELOW;
-#define MI_SMALL_LAUNCH(KWV, PR, SL)                                                             \
+#define MI_SMALL_LAUNCH(KWV, PR, SL, TGV)                                                        \
   do {                                                                                         \
-    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL>), lds)) return; \
-    qmm_small_kernel<BITS, GLU, KWV, PR, SL><<<grid, 256, lds, st>>>(a, tt, sk);               \
+    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV>), lds)) return; \
+    qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV><<<grid, 256, lds, st>>>(a, tt, sk);          \
   } while (0)
-#define MI_SMALL(KWV)                                                                          \
+#define MI_SMALL(KWV, TGV)                                                                     \
   do {                                                                                         \
-    if (slabs) MI_SMALL_LAUNCH(KWV, true, true); /* long rows: few blocks per CU anyway */      \
-    else if (precise) MI_SMALL_LAUNCH(KWV, true, false);                                       \
-    else MI_SMALL_LAUNCH(KWV, false, false);                                                   \
+    if (slabs) MI_SMALL_LAUNCH(KWV, true, true, TGV); /* long rows: few blocks per CU anyway */ \
+    else if (precise) MI_SMALL_LAUNCH(KWV, true, false, TGV);                                  \
+    else MI_SMALL_LAUNCH(KWV, false, false, TGV);                                              \
   } while (0)
-  if (kw == 4) MI_SMALL(4);
-  else if (kw == 2) MI_SMALL(2);
-  else MI_SMALL(1);
+  if constexpr (BITS == 4) {
+    if (two_groups) {
+      MI_SMALL(1, 2);
+      return;
+    }
+  }
+  if (kw == 4) MI_SMALL(4, 1);
+  else if (kw == 2) MI_SMALL(2, 1);
+  else MI_SMALL(1, 1);
 #undef MI_SMALL_LAUNCH
 #undef MI_SMALL
 }

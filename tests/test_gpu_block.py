@@ -116,6 +116,13 @@ def test_tile_classes(orc, T, E, k, bits, zipf):
     _run_case(orc, 256, E, k, 384, bits, T, 0, seed=31 + T, zipf_s=zipf)
 
 
+@pytest.mark.parametrize("T,H,I", [(40, 2048, 768), (44, 1024, 2048), (13, 256, 384), (16, 2048, 256)])
+def test_two_token_groups_per_pass(orc, T, H, I):
+    # 4-bit segments of 9 to 16 rows take one pass of the streaming kernel (two MFMA tiles of 8
+    # tokens against each chunk of weights); rows of 2048 values are staged in slabs of 1024
+    _run_case(orc, H, 8, 2, I, 4, T, 0, seed=91 + T)
+
+
 @pytest.mark.parametrize("T,E,k,zipf", [(100, 16, 2, 1.5), (40, 16, 4, 1.2), (150, 32, 4, 1.0), (150, 32, 4, None)])
 def test_light_batches_tile_only_long_segments(orc, T, E, k, zipf):
     # 6 to 20 rows per expert on average (4-bit): the streamed segments lead on the caller's stream,

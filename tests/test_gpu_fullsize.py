@@ -18,6 +18,8 @@ pytestmark = pytest.mark.gpu
 CASES = [
     # config, tokens, zipf s
     ("qwen3_30b_a3b", 32, None),
+    ("qwen3_30b_a3b", 160, None),   # 10 rows per expert: two token groups per pass, rows staged in slabs of 1024
+    ("qwen3_30b_a3b", 200, 1.1),    # light batch, uneven routing: long segments tiled beside the streamed ones
     ("qwen3_30b_a3b", 4096, 1.1),
     ("mixtral_8x7b", 1, None),
     ("mixtral_8x7b", 16, None),   # streamed; the down product's rows (K = 14336) go through LDS in slabs

@@ -94,27 +94,29 @@ __global__ __launch_bounds__(256) void router_logits_kernel(
 // the four kq lanes of a row cover 32 consecutive h in 8 steps (any K order gives the same sum).
 typedef __attribute__((__vector_size__(4 * sizeof(double)))) double f64x4_t;
 
+// NT: 16-row sub-tiles per side of a block's tile (2: 32 tokens x 32 experts, 1: 16 x 16).
+template <int NT>
 __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg,
     const float *__restrict__ bias, int64_t T, int H, int E, uint16_t *__restrict__ logits) {
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, kq = lane >> 4;
-  const int64_t t0 = (int64_t)blockIdx.x * 32;
-  const int e0 = blockIdx.y * 32;
-  const uint16_t *xr[2], *wr[2];
+  const int64_t t0 = (int64_t)blockIdx.x * (16 * NT);
+  const int e0 = blockIdx.y * (16 * NT);
+  const uint16_t *xr[NT], *wr[NT];
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
+  for (int a = 0; a < NT; ++a) {
     const int64_t t = t0 + 16 * a + i;
     const int e = e0 + 16 * a + i;
     xr[a] = x + (t < T ? t : T - 1) * H + kq * 8;
     wr[a] = wg + (int64_t)(e < E ? e : E - 1) * H + kq * 8;
   }
-  f64x4_t acc[2][2];
+  f64x4_t acc[NT][NT];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < NT; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b) acc[a][b] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+    for (int b = 0; b < NT; ++b) acc[a][b] = f64x4_t{0.0, 0.0, 0.0, 0.0};
 
   // Two register sets take turns: the loads of the next chunk are issued before the current
   // chunk is multiplied and waited for after it.  (Every load is unconditional, its index clamped
@@ -122,32 +124,36 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
   // transparent index lets it fold the prefetch back into the next iteration's top.)
   const int nchunks = H / 32;
   struct Chunk {
-    uint4 x[2], w[2];
+    uint4 x[NT], w[NT];
   };
   auto fetch = [&](int c, Chunk &R) __attribute__((always_inline)) {
     int cc = c < nchunks ? c : nchunks - 1;
     asm volatile("" : "+s"(cc));
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < NT; ++a) {
       R.x[a] = *reinterpret_cast<const uint4 *>(xr[a] + cc * 32);
       R.w[a] = *reinterpret_cast<const uint4 *>(wr[a] + cc * 32);
     }
   };
   auto multiply = [&](const Chunk &R) __attribute__((always_inline)) {
-    const uint32_t xa[2][4] = {{R.x[0].x, R.x[0].y, R.x[0].z, R.x[0].w}, {R.x[1].x, R.x[1].y, R.x[1].z, R.x[1].w}};
-    const uint32_t wb[2][4] = {{R.w[0].x, R.w[0].y, R.w[0].z, R.w[0].w}, {R.w[1].x, R.w[1].y, R.w[1].z, R.w[1].w}};
+    uint32_t xa[NT][4], wb[NT][4];
+#pragma unroll
+    for (int a = 0; a < NT; ++a) {
+      xa[a][0] = R.x[a].x; xa[a][1] = R.x[a].y; xa[a][2] = R.x[a].z; xa[a][3] = R.x[a].w;
+      wb[a][0] = R.w[a].x; wb[a][1] = R.w[a].y; wb[a][2] = R.w[a].z; wb[a][3] = R.w[a].w;
+    }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      double av[2], bv[2];
+      double av[NT], bv[NT];
 #pragma unroll
-      for (int a = 0; a < 2; ++a) {
+      for (int a = 0; a < NT; ++a) {
         av[a] = (double)((s & 1) ? bf16hi_to_f32(xa[a][s >> 1]) : bf16lo_to_f32(xa[a][s >> 1]));
         bv[a] = (double)((s & 1) ? bf16hi_to_f32(wb[a][s >> 1]) : bf16lo_to_f32(wb[a][s >> 1]));
       }
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < NT; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < NT; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[a], bv[b], acc[a][b], 0, 0, 0);
     }
   };
@@ -166,17 +172,18 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
   }
   if (c < nchunks) multiply(r0);  // an odd chunk left over (already fetched)
 
-  __shared__ double part[4][4][4][64];  // [wave][tile][r][lane]
+  __shared__ double part[4][NT * NT][4][64];  // [wave][tile][r][lane]
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < NT; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < NT; ++b)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) part[wave][a * 2 + b][r][lane] = acc[a][b][r];
+      for (int r = 0; r < 4; ++r) part[wave][a * NT + b][r][lane] = acc[a][b][r];
   __syncthreads();
-  // wave w finishes tile w = (a, b) = (w >> 1, w & 1); a lane's register r holds D[4 r + kq][i]
+  // wave w finishes sub-tile w = (a, b) = (w / NT, w % NT); a lane's register r holds D[4 r + kq][i]
   // (fp64 tiles interleave the rows over the four lane groups, unlike the fp32 16x16 layout)
-  const int a = wave >> 1, b = wave & 1;
+  if (wave >= NT * NT) return;
+  const int a = wave / NT, b = wave % NT;
   const int e = e0 + 16 * b + i;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -197,8 +204,16 @@ hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const flo
     dim3 grid((unsigned)T, (unsigned)((E + 3) / 4));
     router_logits_kernel<1, 1><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
   } else {
+    // A block is bound by its CU's fp64 matrix rate whatever its number of waves, so what counts
+    // is the number of blocks: 32 x 32 tiles when they fill the chip, 16 x 16 (four times the
+    // blocks, each a quarter of the work) when they would not (512 tokens x 128 experts: 64 tiles).
     dim3 grid((unsigned)((T + 31) / 32), (unsigned)((E + 31) / 32));
-    router_logits_mfma_kernel<<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+    if ((int64_t)grid.x * grid.y >= 256) {
+      router_logits_mfma_kernel<2><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+    } else {
+      grid = dim3((unsigned)((T + 15) / 16), (unsigned)((E + 15) / 16));
+      router_logits_mfma_kernel<1><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+    }
   }
   return hipGetLastError();
 }

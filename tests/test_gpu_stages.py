@@ -19,6 +19,8 @@ def m():
 @pytest.mark.parametrize("T,H,E,k,mode,bias", [
     (1, 2048, 128, 8, 0, False), (33, 2048, 128, 8, 0, True), (300, 512, 60, 6, 1, False),
     (65, 4096, 8, 2, 2, False), (17, 256, 300, 8, 0, True), (5, 128, 5, 5, 2, False),
+    # 256 and more 32 x 32 logit tiles: the larger tile of the fp64 kernel (fewer: 16 x 16 tiles), ragged edges
+    (2048, 256, 128, 8, 0, True), (1000, 128, 300, 4, 1, False),
 ])
 def test_route_bit_exact(orc, m, T, H, E, k, mode, bias):
     print(f"route T={T} H={H} E={E} k={k} mode={mode}", flush=True)

@@ -198,11 +198,12 @@ def test_graph_replays_equal_eager(orc, T):
         torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("T", [16, 400])
+@pytest.mark.parametrize("T", [16, 40, 70, 400])
 def test_two_handles_on_two_streams(orc, T):
     """Handles are independent: two layers running concurrently on two streams (each with its own
-    workspace) give what they give one after the other.  At 400 tokens each forward also forks its
-    kernel chains onto the handle's own streams and joins them back."""
+    workspace) give what they give one after the other.  From 40 tokens on each forward also forks
+    its kernel chains onto the handle's own streams and joins them back (40 and 70: streamed
+    segments first, with the one-launch router and the separate kernels; 400: tiles first)."""
     import mlx_rs_amd as m
     H, E, k, I = 256, 16, 4, 256
     print(f"two handles T={T}", flush=True)

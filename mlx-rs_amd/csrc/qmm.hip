@@ -84,8 +84,11 @@ extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
 #ifndef MI_MOE_TG2_AVG
 #define MI_MOE_TG2_AVG 5   // rows per active expert from which the 4-bit kernel takes two token groups per pass
 #endif
-#ifndef MI_MOE_TG2_SLAB
-#define MI_MOE_TG2_SLAB 1024
+#ifndef MI_MOE_CUS
+#define MI_MOE_CUS 256  // compute units of an MI355X
+#endif
+#ifndef MI_MOE_SLAB_MIN
+#define MI_MOE_SLAB_MIN 1024  // smallest slab (K values)
 #endif
 #ifndef MI_MOE_PRECISE_BELOW
 #define MI_MOE_PRECISE_BELOW 2  // blocks per CU up to which the ring takes the unconditional form
@@ -108,15 +111,20 @@ struct ChunkRegs {
 // LDS layout of one token tile (all offsets 16-byte aligned):
 //   [0, (tt+1)*xstride)           tt staged activation rows + one all-zero row
 //   then groups x TT fp32         sum of x over each quantisation group, per token slot
-//   then per wave, per tensor     the bf16 scales (and biases) of the wave's 16 weight rows,
-//                                 a flat copy of 16 * K/64 values (they are contiguous in memory)
+//   then per wave, per tensor     the bf16 scales (and biases) of the wave's 16 weight rows: a flat
+//                                 copy of 16 * K/64 values (they are contiguous in memory), or with
+//                                 slabs the slab's sk/64 values of each of the 16 rows
 // xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
 __host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
 __host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }  // 16 rows x K/64 bf16
+// K values the scale / bias tiles in LDS cover: the whole row (fetched once, ahead of everything
+// else) up to K = 4096; beyond, with slabs, the slab (a row of 14336 values has 7 KB of scales and
+// biases per wave and tensor: more than the activations of a few tokens)
+__host__ __device__ constexpr int sb_tile_k(int K, int sk) { return sk < K && K > 4096 ? sk : K; }
 // sk: K values of the activation rows staged at a time (a slab; the whole row when sk = K)
 __host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors) {
   return (size_t)(tt + 1) * x_stride_bytes(sk) + (size_t)(sk / 64) * TT * 4 +
-         (size_t)4 * n_tensors * sb_tile_bytes(K);
+         (size_t)4 * n_tensors * sb_tile_bytes(sb_tile_k(K, sk));
 }
 
 // PRECISE: the ring's refills are issued without a condition (chunk index clamped), so the compiler
@@ -181,7 +189,12 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     br[1] = make_rsrc(a.b1 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
   }
   const uint32_t w_voff = (uint32_t)n * row_bytes + kb * 16;  // lane kb: 16 bytes of the 64-byte chunk
-  const int sbt = sb_tile_bytes(K);
+  // Long rows are staged a slab of sk K values at a time (sk = K: the whole row); the weight
+  // stream, its ring and the accumulators run on across the slabs.
+  const int sk = SLABS ? sk_arg : K;
+  const int groups_per_slab = sk / 64;
+  const bool sb_whole = !SLABS || sb_tile_k(K, sk) == K;  // scale / bias tiles of the whole row, not per slab
+  const int sbt = sb_tile_bytes(sb_tile_k(K, sk));       // bytes of one tensor's scale (bias) tile in LDS
 
   // issue every global load of chunk ch into R
   auto issue = [&](int ch, Regs &R) {
@@ -205,19 +218,17 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   constexpr int SBI = 2;        // 16-byte loads per lane per tensor kept in registers (K <= 4096)
   const uint32_t sb_goff = (uint32_t)n0 * groups_per_row * 2 + lane * 16;
   u32x4_t sbv[NTEN][SBI];
+  if (sb_whole) {
 #pragma unroll
-  for (int t = 0; t < NTEN; ++t)
+    for (int t = 0; t < NTEN; ++t)
 #pragma unroll
-    for (int i = 0; i < SBI; ++i)
-      if (i * 1024 < sbt)
-        sbv[t][i] = __builtin_amdgcn_raw_buffer_load_b128((t & 1) ? br[t >> 1] : sr[t >> 1], sb_goff, i * 1024, 0);
+      for (int i = 0; i < SBI; ++i)
+        if (i * 1024 < sbt)
+          sbv[t][i] = __builtin_amdgcn_raw_buffer_load_b128((t & 1) ? br[t >> 1] : sr[t >> 1], sb_goff, i * 1024, 0);
+  }
 
   MI_STAMP(1);
-  // Long rows are staged a slab of sk K values at a time (sk = K: the whole row); the weight
-  // stream, its ring and the accumulators run on across the slabs.
-  const int sk = SLABS ? sk_arg : K;
   const int xstride = x_stride_bytes(sk);
-  const int groups_per_slab = sk / 64;
   const uint32_t nib_mask = opaque_reg(0x000f000fu), nib_magic = opaque_reg(0x43004300u);  // q -> bf16 128 + q
 
   extern __shared__ __align__(16) unsigned char lds[];
@@ -225,19 +236,37 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   float *lds_gs = reinterpret_cast<float *>(lds + (tt + 1) * xstride);  // [groups of the slab][TTL] sums of x
   unsigned char *lds_sb = lds + (tt + 1) * xstride + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
 
-  // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait)
+  // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait);
+  // long rows in slabs: each slab brings its own piece (see the slab loop)
+  if (sb_whole) {
 #pragma unroll
-  for (int t = 0; t < NTEN; ++t) {
+    for (int t = 0; t < NTEN; ++t) {
 #pragma unroll
-    for (int i = 0; i < SBI; ++i)
-      if (i * 1024 + lane * 16 < sbt)
-        *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + i * 1024 + lane * 16) = sbv[t][i];
-    for (int off = SBI * 1024 + lane * 16; off < sbt; off += 1024)  // K > 4096: the rest, synchronously
-      *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + off) = __builtin_amdgcn_raw_buffer_load_b128(
-          (t & 1) ? br[t >> 1] : sr[t >> 1], (uint32_t)n0 * groups_per_row * 2 + off, 0, 0);
+      for (int i = 0; i < SBI; ++i)
+        if (i * 1024 + lane * 16 < sbt)
+          *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + i * 1024 + lane * 16) = sbv[t][i];
+      for (int off = SBI * 1024 + lane * 16; off < sbt; off += 1024)  // K > 4096: the rest, synchronously
+        *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + off) = __builtin_amdgcn_raw_buffer_load_b128(
+            (t & 1) ? br[t >> 1] : sr[t >> 1], (uint32_t)n0 * groups_per_row * 2 + off, 0, 0);
+    }
   }
-  // this lane's scale / bias of chunk 0: row c, group (4-bit) kb >> 1 of the chunk's two
-  const unsigned char *sbl = lds_sb + (c * groups_per_row + (BITS == 4 ? (kb >> 1) : 0)) * 2;
+  // the scales / biases of the groups [s0 / 64, (s0 + sk) / 64) of the wave's 16 rows: sk / 32 bytes
+  // per row and tensor, in 16-byte pieces (the launcher takes slabs only when rows of scales are
+  // 16-byte aligned, K a multiple of 512).  Past a row's end a piece reads the next row's (or, past
+  // the tensor, zeros): those values belong to no chunk.
+  auto load_sb_slab = [&](int s0) __attribute__((always_inline)) {
+    const int ppr = groups_per_slab / 8;  // pieces per row
+#pragma unroll
+    for (int t = 0; t < NTEN; ++t)
+      for (int p = lane; p < 16 * ppr; p += 64) {
+        const int row = p / ppr, piece = p % ppr;
+        *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + p * 16) = __builtin_amdgcn_raw_buffer_load_b128(
+            (t & 1) ? br[t >> 1] : sr[t >> 1],
+            (uint32_t)(n0 + row) * groups_per_row * 2 + (uint32_t)(s0 / 64) * 2 + piece * 16, 0, 0);
+      }
+  };
+  // this lane's scale / bias of the first chunk in LDS: row c, group (4-bit) kb >> 1 of the chunk's two
+  const unsigned char *sbl = lds_sb + (c * (sb_whole ? groups_per_row : groups_per_slab) + (BITS == 4 ? (kb >> 1) : 0)) * 2;
   __shared__ float red[KW > 1 ? KW : 1][KW > 1 ? NW : 1][NM][4][KW > 1 ? 64 : 1];
 
   // zero row and zero group sums (slots that carry no token stay zero for the whole launch)
@@ -306,7 +335,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
         const float4 xs = *reinterpret_cast<const float4 *>(gsl + (SLABS ? ch - slab_ch0 : ch) * (BITS == 4 ? 2 : 1) * TTL + TT * g);
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-          const int goff = ch * (BITS == 4 ? 4 : 2);
+          const int goff = (sb_whole ? ch : ch - slab_ch0) * (BITS == 4 ? 4 : 2);
           const float sc = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m) * sbt + goff));
           float bi = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m + 1) * sbt + goff));
           if constexpr (BITS == 4) bi = __builtin_fmaf(-128.0f, sc, bi);
@@ -441,6 +470,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
         __syncthreads();  // every wave is done reading the previous slab or tile
         slab_ch0 = s0 / CH;
         if (s0 == 0 && t0 > 0) reprime();
+        if (!sb_whole) load_sb_slab(s0);
         stage_rows(s0, sl);
         __syncthreads();
         after_stage(s0);
@@ -542,9 +572,9 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   if (longest < want) want = (int)longest;
   // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is
   // traded for occupancy only down to about twice the average segment; below that the tile keeps
-  // its rows even if a CU then holds one block.  Rows longer than 4096 values are staged in slabs
-  // of 4096 (2048 if that is what it takes to keep the rows: the scale/bias tiles of a long row
-  // are large too); the weight stream runs on across the slabs.
+  // its rows even if a CU then holds one block.  Long rows are staged in slabs of 4096, 2048 or
+  // 1024 values (activations, their group sums and the scale/bias tiles all shrink with the slab);
+  // the weight stream runs on across the slabs.
   const size_t lds_soft = 60 * 1024, lds_hard = 150 * 1024;  // + up to 8 KB of static LDS (K-split reduction) under the 160 KB of a CU
   const int64_t avg2 = (2 * a.total_rows + a.max_active - 1) / a.max_active;
   const int need = (int)(avg2 < 1 ? 1 : (avg2 < want ? avg2 : want));
@@ -554,19 +584,31 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
     while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, GLU ? 4 : 2) > lds_hard) --t;
     return t;
   };
-  int sk = a.K;  // the whole row if the tokens wanted fit beside it
+  // The whole row, or the largest slab that does better, first in tokens per pass, then in blocks
+  // per CU.  What counts as better in blocks (measured): nothing beyond one, if the launch has no
+  // more blocks than the chip has CUs (Mixtral's down product for one token is 256 blocks: slabs
+  // only cost it barriers); a third block only with up to two slabs per row (sixteen 2048-value
+  // rows in two slabs of 1024: yes; 4096-value rows in four: no); a second block always.  Slabs
+  // need rows of scales that are 16-byte aligned (K a multiple of 512).
+  const int64_t launch_blocks = (int64_t)((a.N + 16 * (4 / kw) - 1) / (16 * (4 / kw))) * a.max_active;
+  auto blocks_of = [&](int slab, int t) {
+    const int b = (int)((size_t)160 * 1024 / small_lds_bytes(a.K, slab, t, TTL, GLU ? 4 : 2));
+    const int cap = launch_blocks <= MI_MOE_CUS ? 1 : (2 * slab >= a.K ? 3 : 2);
+    return b < cap ? b : cap;
+  };
+  int sk = a.K;
   int tt = fit(sk);
-  if (two_groups && MI_MOE_TG2_SLAB > 0 && a.K > MI_MOE_TG2_SLAB && a.K % MI_MOE_TG2_SLAB == 0 &&
-      small_lds_bytes(a.K, sk, tt, TTL, GLU ? 4 : 2) > lds_soft) {
-    // sixteen whole rows leave room for one block per CU: stage them in slabs instead
-    sk = MI_MOE_TG2_SLAB;
-    tt = fit(sk);
-  } else if (tt < need && a.K > 4096) {
-    sk = 4096;
-    tt = fit(sk);
-    if (tt < need && fit(2048) > tt) {
-      sk = 2048;
-      tt = fit(sk);
+  if (a.K % 512 == 0) {
+    int best_t = tt < need ? tt : need, best_b = blocks_of(sk, tt);
+    for (int cand = 4096; cand >= MI_MOE_SLAB_MIN; cand /= 2) {
+      if (cand >= a.K) continue;
+      const int t = fit(cand), tn = t < need ? t : need, b = blocks_of(cand, t);
+      if (tn > best_t || (tn == best_t && b > best_b)) {
+        sk = cand;
+        tt = t;
+        best_t = tn;
+        best_b = b;
+      }
     }
   }
   const bool slabs = sk < a.K;

@@ -22,7 +22,8 @@ CASES = [
     ("qwen3_30b_a3b", 200, 1.1),    # light batch, uneven routing: long segments tiled beside the streamed ones
     ("qwen3_30b_a3b", 4096, 1.1),
     ("mixtral_8x7b", 1, None),
-    ("mixtral_8x7b", 16, None),   # streamed; the down product's rows (K = 14336) go through LDS in slabs
+    ("mixtral_8x7b", 4, None),    # streamed; the down product's rows (K = 14336) and their scales go through LDS in slabs
+    ("mixtral_8x7b", 16, None),
     ("mixtral_8x7b", 64, None),   # 64-row tiles
     ("mixtral_8x7b", 2048, None),
     ("qwen3_235b_a22b", 8192, 1.3),

@@ -19,11 +19,11 @@ constexpr int kWave = 64;
 #define MI_TMR4 9
 #define MI_TMR8 9
 #define MI_TAVG4 20
-#define MI_TAVG8 12
+#define MI_TAVG8 20
 #endif
 #ifndef MI_TLIGHT4
 #define MI_TLIGHT4 6
-#define MI_TLIGHT8 12
+#define MI_TLIGHT8 20
 #define MI_TMRL4 17
 #define MI_TMRL8 9
 #endif

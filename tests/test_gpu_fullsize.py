@@ -24,7 +24,8 @@ CASES = [
     ("mixtral_8x7b", 1, None),
     ("mixtral_8x7b", 4, None),    # streamed; the down product's rows (K = 14336) and their scales go through LDS in slabs
     ("mixtral_8x7b", 16, None),
-    ("mixtral_8x7b", 64, None),   # 64-row tiles
+    ("mixtral_8x7b", 64, None),   # streamed, 16 rows per expert
+    ("mixtral_8x7b", 96, None),   # 64-row tiles
     ("mixtral_8x7b", 2048, None),
     ("qwen3_235b_a22b", 8192, 1.3),
 ]

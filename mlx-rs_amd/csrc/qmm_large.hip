@@ -74,7 +74,7 @@ constexpr size_t large_lds_bytes(int bm) { return (size_t)2 * (bm + BR) * LDR * 
 // bound by that dequantisation, which is still far cheaper than streaming the weights once per
 // 8 tokens.
 template <int BITS, bool GLU, int MT>
-__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT == 4 ? 2 : 4))) void qmm_large_kernel(GroupedArgs a, const uint32_t *__restrict__ tiles, int n_ntiles, int cap, int chunk) {
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT == 4 ? 2 : 4))) void qmm_large_kernel(GroupedArgs a, const uint32_t *__restrict__ tiles, int n_ntiles, int cap, int chunk, int sub_log2) {
   constexpr int NI = GLU ? 128 : 256;  // distinct output columns per block
   constexpr int BM = 64 * MT;          // token rows per block
   constexpr int NA = MT >= 2 ? MT / 2 : 1;  // 16-byte activation loads per thread and step
@@ -85,23 +85,29 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
   // whole tiles per XCD would leave XCDs idle (one M tile of a 14336-wide GLU is 112 blocks, all on
   // one XCD's 32 CUs), so the N tiles of an M tile are dealt over the XCDs in chunks of `chunk`.
   // Both candidate records are fetched along with the count (indices clamped to the list's capacity).
+  // sub_log2 > 0: the list's tiles are larger than this kernel's; each is taken as 2 or 4 M tiles of
+  // BM rows (the launcher does that when even so the chip has blocks to spare: a 64-row block's
+  // K step is shorter than a 256-row block's).
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int n_chunks = (n_ntiles + chunk - 1) / chunk;
   const uint32_t whole_id = (uint32_t)(j / n_ntiles) * 8u + xcd;
   const uint32_t unit = (uint32_t)(j / chunk) * 8u + xcd;
   const uint32_t spread_id = unit / (uint32_t)n_chunks;
   const uint4 *const recs = reinterpret_cast<const uint4 *>(tiles) + 1;
-  const uint4 rec_whole = recs[whole_id < (uint32_t)cap ? whole_id : (uint32_t)cap - 1u];
-  const uint4 rec_spread = recs[spread_id < (uint32_t)cap ? spread_id : (uint32_t)cap - 1u];
-  const uint32_t n_mtiles = tiles[0];
+  const uint32_t whole_rec = whole_id >> sub_log2, spread_rec = spread_id >> sub_log2;
+  const uint4 rec_whole = recs[whole_rec < (uint32_t)cap ? whole_rec : (uint32_t)cap - 1u];
+  const uint4 rec_spread = recs[spread_rec < (uint32_t)cap ? spread_rec : (uint32_t)cap - 1u];
+  const uint32_t n_mtiles = tiles[0] << sub_log2;
   const bool spread = n_mtiles < (uint32_t)kSpreadBelow;
   const uint32_t mt_id = spread ? spread_id : whole_id;
   const int nt = spread ? (int)(unit % (uint32_t)n_chunks) * chunk + j % chunk : j % n_ntiles;
   const uint4 rec = spread ? rec_spread : rec_whole;
   if (mt_id >= n_mtiles || nt >= n_ntiles) return;
+  const int part = (int)(mt_id & ((1u << sub_log2) - 1u)) * BM;  // first row of this block's piece of the tile
   const int e = (int)rec.x;
-  const int64_t row0 = rec.y;
-  const int rows = (int)rec.z;
+  const int64_t row0 = (int64_t)rec.y + part;
+  const int rows = (int)rec.z - part < BM ? (int)rec.z - part : BM;
+  if (rows <= 0) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -399,7 +405,8 @@ hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *ou
 }
 
 template <int BITS, bool GLU, int MT>
-static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int cap, hipStream_t st) {
+static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int list_cap, int sub_log2, hipStream_t st) {
+  const int cap = list_cap << sub_log2;  // M tiles of this kernel's size
   const int ni = GLU ? 128 : 256;
   const int n_ntiles = (a.N + ni - 1) / ni;
   // ids for either dealing of the tiles (see the kernel): whole M tiles per XCD, or chunks of an
@@ -423,18 +430,39 @@ static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int ca
       return e;
     if (dev >= 0 && dev < kMaxDevices) raised[dev].store(true, std::memory_order_release);
   }
-  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles, cap, chunk);
+  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles, list_cap, chunk, sub_log2);
   return hipGetLastError();
 }
 
 // class 0 / 1 / 2 = the 256- / 128- / 64-row tile list.  A segment is at most max_rows_per_expert
-// long: a class that cannot occur is not launched.
+// long: a class that cannot occur is not launched.  When even 64-row (128-row) tiles throughout
+// could not give the chip more than MI_FEW_BLOCKS blocks, one per CU (few experts, a narrow output:
+// Mixtral's down product at a few hundred tokens is a few dozen 256-row blocks of 448 K steps each,
+// bound by the length of a step), the larger lists are run by the smaller kernel, 2 or 4 blocks
+// per tile (measured: 256 / 512 tokens of that shape -5 / -6 %; with a bound of 384 or 512 blocks
+// other batch sizes gain 3 % and 512 tokens lose 6 %).
+#ifndef MI_FEW_BLOCKS
+#define MI_FEW_BLOCKS 256
+#endif
 template <int BITS, bool GLU>
 static hipError_t launch_class(const GroupedArgs &a, int cls, hipStream_t st) {
   const uint32_t *const list = tile_list(a.mtiles, cls, a.max_mtiles, a.tile_cap_e);
-  if (cls == 0) return a.max_rows_per_expert > 128 ? launch_one<BITS, GLU, 4>(a, list, a.max_mtiles, st) : hipSuccess;
-  if (cls == 1) return a.max_rows_per_expert > 64 ? launch_one<BITS, GLU, 2>(a, list, a.tile_cap_e, st) : hipSuccess;
-  return launch_one<BITS, GLU, 1>(a, list, a.tile_cap_e, st);
+  const int ni = GLU ? 128 : 256;
+  const int64_t n_ntiles = (a.N + ni - 1) / ni;
+  auto blocks_with = [&](int rows_per_tile) { return (a.total_rows / rows_per_tile + a.max_active) * n_ntiles; };
+  const int mt_max = blocks_with(64) <= MI_FEW_BLOCKS ? 1 : (blocks_with(128) <= MI_FEW_BLOCKS ? 2 : 4);
+  if (cls == 0) {
+    if (a.max_rows_per_expert <= 128) return hipSuccess;
+    if (mt_max == 1) return launch_one<BITS, GLU, 1>(a, list, a.max_mtiles, 2, st);
+    if (mt_max == 2) return launch_one<BITS, GLU, 2>(a, list, a.max_mtiles, 1, st);
+    return launch_one<BITS, GLU, 4>(a, list, a.max_mtiles, 0, st);
+  }
+  if (cls == 1) {
+    if (a.max_rows_per_expert <= 64) return hipSuccess;
+    if (mt_max == 1) return launch_one<BITS, GLU, 1>(a, list, a.tile_cap_e, 1, st);
+    return launch_one<BITS, GLU, 2>(a, list, a.tile_cap_e, 0, st);
+  }
+  return launch_one<BITS, GLU, 1>(a, list, a.tile_cap_e, 0, st);
 }
 
 bool large_qmm_applies(const GroupedArgs &a) { return a.mtiles && a.tile_cap_e > 0 && a.x_perm; }

@@ -9,10 +9,10 @@ from helpers import (assert_close_bf16, bits_u16, bits_u32, bf16_tensor, device_
 pytestmark = pytest.mark.gpu
 
 
-def _run_case(orc, H, E, k, I, bits, T, score_mode, seed=0, zipf_s=None, threads=16):
+def _run_case(orc, H, E, k, I, bits, T, score_mode, seed=0, zipf_s=None, threads=16, std=0.02):
     import mlx_rs_amd as m
     print(f"case H={H} E={E} k={k} I={I} bits={bits} T={T} mode={score_mode} seed={seed}", flush=True)
-    W = host_layer(orc, H, E, k, I, bits, seed, zipf_s=zipf_s)
+    W = host_layer(orc, H, E, k, I, bits, seed, std=std, zipf_s=zipf_s)
     x = host_tokens(orc, T, H, seed)
     cfg = m.MoeConfig(H, E, k, I, bits, 64, score_mode)
     blk = device_block(m, cfg, W)
@@ -114,6 +114,15 @@ def test_tile_classes(orc, T, E, k, bits, zipf):
     # segments of 9 rows and more are cut into 256-, 128- and 64-row tiles, shorter ones stream:
     # these shapes put segments into every class, with remainders on both sides of each boundary
     _run_case(orc, 256, E, k, 384, bits, T, 0, seed=31 + T, zipf_s=zipf)
+
+
+@pytest.mark.parametrize("bits,zipf", [(4, None), (8, 0.7)])
+def test_tile_classes_with_the_chip_full(orc, bits, zipf):
+    # narrow layers leave the chip blocks to spare and run their 256- and 128-row tiles with the
+    # 64-row kernel (the shapes of test_tile_classes); here both products have more than 256 blocks
+    # even with 128-row tiles, so each list is run by the kernel of its own size (weights of half the
+    # usual spread: the absolute bar is meant for outputs of magnitude 1, these rows are 3072 long)
+    _run_case(orc, 3072, 8, 2, 1536, bits, 1100, 0, seed=17 + bits, zipf_s=zipf, std=0.01)
 
 
 @pytest.mark.parametrize("T,H,I", [(40, 2048, 768), (44, 1024, 2048), (13, 256, 384), (16, 2048, 256)])

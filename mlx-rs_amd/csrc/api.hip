@@ -314,19 +314,28 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     // segment in a heavy batch, the streamed segments of a light one (whose tile lists are empty
     // unless the routing is uneven; the copy of x with paired rows, which only the tiles read,
     // then runs on a side stream as well).
+    // A segment is at most T rows long: a class that cannot occur gets no stream (a fork and a
+    // join cost a few microseconds each).
+    const bool exists[4] = {T > 128, T > 64, true, true};
+    int n_side = 0;
     MI_HIP(hipEventRecord(h->fork, st));
-    for (int i = 0; i < 3; ++i) MI_HIP(hipStreamWaitEvent(h->side[i], h->fork, 0));
     if (streamed_first) {
       MI_HIP(launch_small_qmm(a, true, st));
       MI_HIP(launch_small_qmm(d, false, st));
-      if (paired) {
-        MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, h->side[0]));
-        MI_HIP(hipEventRecord(h->paired, h->side[0]));
-        for (int i = 1; i < 3; ++i) MI_HIP(hipStreamWaitEvent(h->side[i], h->paired, 0));
-      }
       for (int cls = 0; cls < 3; ++cls) {
-        MI_HIP(launch_large_qmm_class(a, true, cls, h->side[cls]));
-        MI_HIP(launch_large_qmm_class(d, false, cls, h->side[cls]));
+        if (!exists[cls]) continue;
+        hipStream_t s = h->side[n_side++];
+        if (n_side == 1) {
+          MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
+          if (paired) {
+            MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, s));
+            MI_HIP(hipEventRecord(h->paired, s));
+          }
+        } else {
+          MI_HIP(hipStreamWaitEvent(s, paired ? h->paired : h->fork, 0));
+        }
+        MI_HIP(launch_large_qmm_class(a, true, cls, s));
+        MI_HIP(launch_large_qmm_class(d, false, cls, s));
       }
     } else {
       // which class is the longest depends on the routing, which the host does not see; it takes
@@ -334,10 +343,14 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
       // -9 % against always leading with the 256-row class; zipf-1.1 routing: +4 to +6 % there)
       const int64_t avg_rows = P / (max_active > 0 ? max_active : 1);
       const int lead = avg_rows <= 64 ? 2 : (avg_rows <= 128 ? 1 : 0);
-      int next_side = 0;
       for (int i = 0; i < 4; ++i) {
         const int chain = i == 0 ? lead : (i <= lead ? i - 1 : i);
-        hipStream_t s = i == 0 ? st : h->side[next_side++];
+        if (!exists[chain]) continue;
+        hipStream_t s = st;
+        if (i > 0) {
+          s = h->side[n_side++];
+          MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
+        }
         if (chain < 3) {
           MI_HIP(launch_large_qmm_class(a, true, chain, s));
           MI_HIP(launch_large_qmm_class(d, false, chain, s));
@@ -347,7 +360,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
         }
       }
     }
-    for (int i = 0; i < 3; ++i) {
+    for (int i = 0; i < n_side; ++i) {
       MI_HIP(hipEventRecord(h->join[i], h->side[i]));
       MI_HIP(hipStreamWaitEvent(st, h->join[i], 0));
     }

@@ -27,7 +27,7 @@
  *    forwards through one handle must not overlap on the GPU (use one stream per handle):
  *    a handle owns 260 bytes of device memory (arrival counters of the decode router
  *    kernel) and three streams with five events (default priority; a forward with an
- *    average of 6 rows per expert or more (20 with 8-bit weights) forks its independent
+ *    average of 6 rows per expert or more (17 with 8-bit weights) forks its independent
  *    kernel chains onto them from `stream` and joins them back before it returns, which is
  *    also what a graph capture of `stream` records), all
  *    created by mi_moe_create on the current device and released by mi_moe_destroy.  No

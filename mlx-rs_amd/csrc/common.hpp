@@ -17,15 +17,15 @@ constexpr int kWave = 64;
 // lists are not built.  Measured crossovers: see the design notes.
 #ifndef MI_TMR4
 #define MI_TMR4 9
-#define MI_TMR8 9
+#define MI_TMR8 17
 #define MI_TAVG4 20
-#define MI_TAVG8 20
+#define MI_TAVG8 17
 #endif
 #ifndef MI_TLIGHT4
 #define MI_TLIGHT4 6
-#define MI_TLIGHT8 20
+#define MI_TLIGHT8 17
 #define MI_TMRL4 17
-#define MI_TMRL8 9
+#define MI_TMRL8 17
 #endif
 __host__ __device__ constexpr int tile_min_rows(int bits, bool heavy) {
   return bits == 4 ? (heavy ? MI_TMR4 : MI_TMRL4) : (heavy ? MI_TMR8 : MI_TMRL8);

@@ -319,51 +319,62 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     const bool exists[4] = {T > 128, T > 64, true, true};
     int n_side = 0;
     MI_HIP(hipEventRecord(h->fork, st));
-    if (streamed_first) {
-      MI_HIP(launch_small_qmm(a, true, st));
-      MI_HIP(launch_small_qmm(d, false, st));
-      for (int cls = 0; cls < 3; ++cls) {
-        if (!exists[cls]) continue;
-        hipStream_t s = h->side[n_side++];
-        if (n_side == 1) {
-          MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
-          if (paired) {
-            MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, s));
-            MI_HIP(hipEventRecord(h->paired, s));
+    // the launches, in a function of their own: whatever happens in it, the side streams it has
+    // used are joined back below (a caller must never be left with work of ours running beside
+    // its stream, or with a capture that has not been joined)
+    auto launch_chains = [&]() -> int {
+      if (streamed_first) {
+        MI_HIP(launch_small_qmm(a, true, st));
+        MI_HIP(launch_small_qmm(d, false, st));
+        for (int cls = 0; cls < 3; ++cls) {
+          if (!exists[cls]) continue;
+          hipStream_t s = h->side[n_side++];
+          if (n_side == 1) {
+            MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
+            if (paired) {
+              MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, s));
+              MI_HIP(hipEventRecord(h->paired, s));
+            }
+          } else {
+            MI_HIP(hipStreamWaitEvent(s, paired ? h->paired : h->fork, 0));
           }
-        } else {
-          MI_HIP(hipStreamWaitEvent(s, paired ? h->paired : h->fork, 0));
+          MI_HIP(launch_large_qmm_class(a, true, cls, s));
+          MI_HIP(launch_large_qmm_class(d, false, cls, s));
         }
-        MI_HIP(launch_large_qmm_class(a, true, cls, s));
-        MI_HIP(launch_large_qmm_class(d, false, cls, s));
-      }
-    } else {
-      // which class is the longest depends on the routing, which the host does not see; it takes
-      // the class of the average segment (even routing: 320 to 2048 tokens of the 128-expert shape
-      // -9 % against always leading with the 256-row class; zipf-1.1 routing: +4 to +6 % there)
-      const int64_t avg_rows = P / (max_active > 0 ? max_active : 1);
-      const int lead = avg_rows <= 64 ? 2 : (avg_rows <= 128 ? 1 : 0);
-      for (int i = 0; i < 4; ++i) {
-        const int chain = i == 0 ? lead : (i <= lead ? i - 1 : i);
-        if (!exists[chain]) continue;
-        hipStream_t s = st;
-        if (i > 0) {
-          s = h->side[n_side++];
-          MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
-        }
-        if (chain < 3) {
-          MI_HIP(launch_large_qmm_class(a, true, chain, s));
-          MI_HIP(launch_large_qmm_class(d, false, chain, s));
-        } else {
-          MI_HIP(launch_small_qmm(a, true, s));
-          MI_HIP(launch_small_qmm(d, false, s));
+      } else {
+        // which class is the longest depends on the routing, which the host does not see; it takes
+        // the class of the average segment (even routing: 320 to 2048 tokens of the 128-expert shape
+        // -9 % against always leading with the 256-row class; zipf-1.1 routing: +4 to +6 % there)
+        const int64_t avg_rows = P / (max_active > 0 ? max_active : 1);
+        const int lead = avg_rows <= 64 ? 2 : (avg_rows <= 128 ? 1 : 0);
+        for (int i = 0; i < 4; ++i) {
+          const int chain = i == 0 ? lead : (i <= lead ? i - 1 : i);
+          if (!exists[chain]) continue;
+          hipStream_t s = st;
+          if (i > 0) {
+            s = h->side[n_side++];
+            MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
+          }
+          if (chain < 3) {
+            MI_HIP(launch_large_qmm_class(a, true, chain, s));
+            MI_HIP(launch_large_qmm_class(d, false, chain, s));
+          } else {
+            MI_HIP(launch_small_qmm(a, true, s));
+            MI_HIP(launch_small_qmm(d, false, s));
+          }
         }
       }
-    }
+      return 0;
+    };
+    const int rc = launch_chains();
+    hipError_t je = hipSuccess;
     for (int i = 0; i < n_side; ++i) {
-      MI_HIP(hipEventRecord(h->join[i], h->side[i]));
-      MI_HIP(hipStreamWaitEvent(st, h->join[i], 0));
+      hipError_t e = hipEventRecord(h->join[i], h->side[i]);
+      if (e == hipSuccess) e = hipStreamWaitEvent(st, h->join[i], 0);
+      if (e != hipSuccess && je == hipSuccess) je = e;
     }
+    if (rc) return rc;
+    MI_HIP(je);
   } else {
     MI_HIP(launch_grouped_qmm(a, true, st));
     MI_STAGE_DONE();

@@ -90,6 +90,9 @@ extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
 #ifndef MI_MOE_SLAB_MIN
 #define MI_MOE_SLAB_MIN 1024  // smallest slab (K values)
 #endif
+#ifndef MI_MOE_SHORT_TT
+#define MI_MOE_SHORT_TT 4  // token rows staged per pass at least, when segments are short on average
+#endif
 #ifndef MI_MOE_PRECISE_BELOW
 #define MI_MOE_PRECISE_BELOW 2  // blocks per CU up to which the ring takes the unconditional form
 #endif
@@ -109,13 +112,17 @@ struct ChunkRegs {
 };
 
 // LDS layout of one token tile (all offsets 16-byte aligned):
-//   [0, (tt+1)*xstride)           tt staged activation rows + one all-zero row
+//   [0, tt*xstride + zero_bytes)  tt staged activation rows + zeros (see zero_bytes)
 //   then groups x TT fp32         sum of x over each quantisation group, per token slot
 //   then per wave, per tensor     the bf16 scales (and biases) of the wave's 16 weight rows: a flat
 //                                 copy of 16 * K/64 values (they are contiguous in memory), or with
 //                                 slabs the slab's sk/64 values of each of the 16 rows
 // xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
 __host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
+// Zeros that lanes without a token read.  Gate/up kernel (long rows, LDS decides how many blocks a
+// CU holds): 64 bytes, read with a chunk stride of zero.  Down kernel: a whole zero row at the common
+// stride (the per-lane stride costs it 6 VGPRs, which would take it from 6 to 5 waves per SIMD).
+__host__ __device__ constexpr int zero_bytes(int sk, bool glu) { return glu ? 64 : 2 * sk + 16; }
 __host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }  // 16 rows x K/64 bf16
 // K values the scale / bias tiles in LDS cover: the whole row (fetched once, ahead of everything
 // else) up to K = 4096; beyond, with slabs, the slab (a row of 14336 values has 7 KB of scales and
@@ -123,7 +130,7 @@ __host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }
 __host__ __device__ constexpr int sb_tile_k(int K, int sk) { return sk < K && K > 4096 ? sk : K; }
 // sk: K values of the activation rows staged at a time (a slab; the whole row when sk = K)
 __host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors) {
-  return (size_t)(tt + 1) * x_stride_bytes(sk) + (size_t)(sk / 64) * TT * 4 +
+  return (size_t)tt * x_stride_bytes(sk) + zero_bytes(sk, n_tensors == 4) + (size_t)(sk / 64) * TT * 4 +
          (size_t)4 * n_tensors * sb_tile_bytes(sb_tile_k(K, sk));
 }
 
@@ -233,8 +240,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
   extern __shared__ __align__(16) unsigned char lds[];
   unsigned char *lds_x = lds;
-  float *lds_gs = reinterpret_cast<float *>(lds + (tt + 1) * xstride);  // [groups of the slab][TTL] sums of x
-  unsigned char *lds_sb = lds + (tt + 1) * xstride + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
+  float *lds_gs = reinterpret_cast<float *>(lds + tt * xstride + zero_bytes(sk, GLU));  // [groups of the slab][TTL] sums of x
+  unsigned char *lds_sb = lds + tt * xstride + zero_bytes(sk, GLU) + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
 
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait);
   // long rows in slabs: each slab brings its own piece (see the slab loop)
@@ -269,8 +276,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   const unsigned char *sbl = lds_sb + (c * (sb_whole ? groups_per_row : groups_per_slab) + (BITS == 4 ? (kb >> 1) : 0)) * 2;
   __shared__ float red[KW > 1 ? KW : 1][KW > 1 ? NW : 1][NM][4][KW > 1 ? 64 : 1];
 
-  // zero row and zero group sums (slots that carry no token stay zero for the whole launch)
-  for (int i = threadIdx.x; i < xstride / 16; i += 256)
+  // zero block and zero group sums (slots that carry no token stay zero for the whole launch)
+  for (int i = threadIdx.x; i < zero_bytes(sk, GLU) / 16; i += 256)
     *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
   for (int i = threadIdx.x; i < groups_per_slab * TTL / 4; i += 256)
     *reinterpret_cast<uint4 *>(lds_gs + i * 4) = make_uint4(0, 0, 0, 0);
@@ -280,6 +287,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
     // set after a slab has been staged (kept out of the staging's way: they cost registers there)
     const unsigned char *xl[TG];  // activation row of this lane (A operand), per token group
+    int xcs[TG];                  // bytes from one chunk of it to the next (0: the zero block)
     const float *gsl;             // group sums of x for this lane's 4 D rows (token slots), first group of the slab
     f32x4_t tot[TG][NM];
     int slab_ch0 = 0;  // first chunk of the slab that is in LDS
@@ -292,7 +300,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
         if (TG > 1 && g > 0) __builtin_amdgcn_sched_barrier(0);
         uint4 xv[XV];
 #pragma unroll
-        for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl[g] + (SLABS ? ch - slab_ch0 : ch) * CH * 2 + i * 16);
+        for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl[g] + (SLABS ? ch - slab_ch0 : ch) * (GLU ? xcs[g] : CH * 2) + i * 16);
         f32x4_t acc[NM];
 #pragma unroll
         for (int m = 0; m < NM; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -400,13 +408,18 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     // after a slab has been staged: where this lane reads, and (first slab) zero accumulators
     auto after_stage = [&](int s0) __attribute__((always_inline)) {
       {
-        // lanes without data read the zero row
+        // lanes without data read zeros (gate/up: the zero block, with a chunk stride of zero)
 #pragma unroll
         for (int g = 0; g < TG; ++g) {
           const int ts_l = (BITS == 4 ? (c & 7) : c) + TT * g;
           bool a_on = ts_l < nt;
           if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
-          xl[g] = lds_x + (a_on ? ts_l : tt) * xstride + kb * (CH / 4) * 2;
+          if constexpr (GLU) {
+            xl[g] = a_on ? lds_x + ts_l * xstride + kb * (CH / 4) * 2 : lds_x + tt * xstride;
+            xcs[g] = a_on ? CH * 2 : 0;
+          } else {
+            xl[g] = lds_x + (a_on ? ts_l : tt) * xstride + kb * (CH / 4) * 2;
+          }
         }
         gsl = lds_gs + (BITS == 4 ? (kb >> 1) * TTL + 4 * (kb & 1) : 4 * kb);
         if (!SLABS || s0 == 0) {
@@ -567,8 +580,10 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int TTL = two_groups ? 2 * TT : TT;  // token slots of one pass
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
   int want = TTL;
-  // short segments on average: stage fewer rows, the LDS saved buys a fourth block per CU
-  if (a.total_rows <= 3 * (int64_t)a.max_active && want > 4) want = 4;
+  // short segments on average: stage fewer rows where the LDS saved buys a fourth block per CU (but
+  // no fewer than that takes: a segment longer than the tile reads its expert's weights again)
+  if (a.total_rows <= 3 * (int64_t)a.max_active)
+    while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, GLU ? 4 : 2) > (size_t)160 * 1024) --want;
   if (longest < want) want = (int)longest;
   // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is
   // traded for occupancy only down to about twice the average segment; below that the tile keeps

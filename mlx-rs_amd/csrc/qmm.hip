@@ -211,7 +211,29 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     }
   };
 
-  // the weight stream does not depend on the tokens: start it before anything else
+  // The first token row this wave stages (row `wave` of the segment): its loads go out ahead of the
+  // weight stream.  Loads come back in the order of issue, so behind the ring's first chunks the
+  // staging would wait for those too, with nothing further in flight meanwhile.  Whole rows of up
+  // to 2048 values (one 16-byte piece per lane and load, four loads).  Not in the gate/up kernel:
+  // there it gains half a microsecond when the chip holds all blocks of the launch at once and
+  // loses two when it does not (a block then starts while others stream; measured).
+  constexpr bool PRE = !SLABS && !GLU;
+  const bool pre_on = PRE && K <= 2048 && wave < cnt && wave < tt;
+  uint4 pre[4];
+  if (PRE && pre_on) {
+    int64_t src = r0 + wave;
+    if (rec_src) src = a.work[(size_t)blockIdx.y * 16 + 4 + wave];
+    else if (a.src_rows) src = a.src_rows[src];
+    const uint16_t *xr = a.x + src * K;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int blk = j * 64 + lane;
+      pre[j] = make_uint4(0, 0, 0, 0);
+      if (blk < K / 8) pre[j] = *reinterpret_cast<const uint4 *>(xr + blk * 8);
+    }
+  }
+
+  // the weight stream does not depend on the tokens either
   Regs ring[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) {
@@ -245,6 +267,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait);
   // long rows in slabs: each slab brings its own piece (see the slab loop)
+  auto park_sb = [&]() __attribute__((always_inline)) {
   if (sb_whole) {
 #pragma unroll
     for (int t = 0; t < NTEN; ++t) {
@@ -257,6 +280,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
             (t & 1) ? br[t >> 1] : sr[t >> 1], (uint32_t)n0 * groups_per_row * 2 + off, 0, 0);
     }
   }
+  };
+  if constexpr (!PRE) park_sb();
   // the scales / biases of the groups [s0 / 64, (s0 + sk) / 64) of the wave's 16 rows: sk / 32 bytes
   // per row and tensor, in 16-byte pieces (the launcher takes slabs only when rows of scales are
   // 16-byte aligned, K a multiple of 512).  Past a row's end a piece reads the next row's (or, past
@@ -281,6 +306,36 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
   for (int i = threadIdx.x; i < groups_per_slab * TTL / 4; i += 256)
     *reinterpret_cast<uint4 *>(lds_gs + i * 4) = make_uint4(0, 0, 0, 0);
+
+  // the prefetched row into LDS, as stage_rows() below does it for the others
+  auto put_row = [&](int ts, int b0, int sl, const uint4 (&v)[4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int blk = b0 + j * 64 + lane;
+      const uint4 w = v[j];
+      float sum = ((bf16lo_to_f32(w.x) + bf16hi_to_f32(w.x)) + (bf16lo_to_f32(w.y) + bf16hi_to_f32(w.y))) +
+                  ((bf16lo_to_f32(w.z) + bf16hi_to_f32(w.z)) + (bf16lo_to_f32(w.w) + bf16hi_to_f32(w.w)));
+      sum += __shfl_xor(sum, 1, kWave);
+      sum += __shfl_xor(sum, 2, kWave);
+      sum += __shfl_xor(sum, 4, kWave);
+      if (blk < sl / 8) {
+        uint4 p = w;
+        if (BITS == 4 && !a.x_paired) {
+          p.x = (w.x & 0xffffu) | (w.z << 16);
+          p.y = (w.x >> 16) | (w.z & 0xffff0000u);
+          p.z = (w.y & 0xffffu) | (w.w << 16);
+          p.w = (w.y >> 16) | (w.w & 0xffff0000u);
+        }
+        *reinterpret_cast<uint4 *>(lds_x + ts * xstride + blk * 16) = p;
+        if ((blk & 7) == 0) lds_gs[(blk >> 3) * TTL + ts] = sum;
+      }
+    }
+  };
+  if constexpr (PRE) {
+    __syncthreads();  // zero fill done
+    if (pre_on) put_row(wave, 0, K, pre);
+    park_sb();
+  }
 
   for (int t0 = 0; t0 < cnt; t0 += tt) {
     const int nt = cnt - t0 < tt ? cnt - t0 : tt;  // tokens of this tile
@@ -367,7 +422,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
           lds_gs[(i / (tt - nt)) * TTL + nt + i % (tt - nt)] = 0.f;
       // wave w stages token slots w, w+4, ...: the source row is wave-uniform (read from the
       // record through the scalar cache) and every load of a row is issued before the first use
-      for (int ts = wave; ts < nt; ts += 4) {
+      for (int ts = wave + (PRE && t0 == 0 && pre_on ? 4 : 0); ts < nt; ts += 4) {
         const int64_t r = r0 + t0 + ts;
         int64_t src = r;
         if (rec_src && t0 + ts < 12) src = a.work[(size_t)blockIdx.y * 16 + 4 + t0 + ts];
@@ -469,7 +524,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
       }
     };
     if constexpr (!SLABS) {
-      __syncthreads();  // zero fill done / every wave is done reading the previous tile
+      if (!PRE || t0 > 0) __syncthreads();  // zero fill done / every wave is done reading the previous tile
       if (t0 > 0) reprime();
       stage_rows(0, K);
       MI_STAMP(2);

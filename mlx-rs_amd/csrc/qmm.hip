@@ -90,6 +90,9 @@ extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
 #ifndef MI_MOE_SLAB_MIN
 #define MI_MOE_SLAB_MIN 1024  // smallest slab (K values)
 #endif
+#ifndef MI_MOE_SHORT_AVG2
+#define MI_MOE_SHORT_AVG2 3  // twice the rows per expert on average up to which segments count as short
+#endif
 #ifndef MI_MOE_SHORT_TT
 #define MI_MOE_SHORT_TT 4  // token rows staged per pass at least, when segments are short on average
 #endif
@@ -637,7 +640,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   int want = TTL;
   // short segments on average: stage fewer rows where the LDS saved buys a fourth block per CU (but
   // no fewer than that takes: a segment longer than the tile reads its expert's weights again)
-  if (a.total_rows <= 3 * (int64_t)a.max_active)
+  if (2 * a.total_rows <= MI_MOE_SHORT_AVG2 * (int64_t)a.max_active)
     while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, GLU ? 4 : 2) > (size_t)160 * 1024) --want;
   if (longest < want) want = (int)longest;
   // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is

@@ -81,6 +81,9 @@ extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
 #ifndef MI_MOE_RING
 #define MI_MOE_RING 4
 #endif
+#ifndef MI_MOE_RING_DEEP
+#define MI_MOE_RING_DEEP 8  // chunks in flight per wave where a CU holds two blocks (registers are plentiful there)
+#endif
 #ifndef MI_MOE_TG2_AVG
 #define MI_MOE_TG2_AVG 5   // rows per active expert from which the 4-bit kernel takes two token groups per pass
 #endif
@@ -148,15 +151,17 @@ __host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int 
 // tokens for the chunk's second quantisation group); with TG = 2 a chunk of weights is multiplied
 // with two such tiles, tokens 0-7 and 8-15 of the pass, before its ring slot is refilled: segments
 // of 9 to 16 rows then take one pass over the expert's weights instead of two.
-template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8)))
+// D: chunks kept in flight per wave (ring depth).  Where a CU holds two blocks a wave may use 256
+// registers, and with 8-bit codes eight chunks in flight instead of four make up for the few waves.
+template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG, int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D > MI_MOE_RING ? 2 : 3, 8)))
 void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   static_assert(TG == 1 || (TG == 2 && BITS == 4 && KW == 1), "two token groups: 4-bit, K not split over waves");
   constexpr int NW = 4 / KW;                    // row tiles per block
   constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one 16-byte load per lane)
   constexpr int XV = BITS == 4 ? 4 : 2;         // 16-byte pieces of activations per lane per chunk
   constexpr int NM = GLU ? 2 : 1;
-  constexpr int D = MI_MOE_RING;                // chunks kept in flight per wave
+  static_assert(D == MI_MOE_RING || PRECISE, "the deep ring goes with unconditional refills");
   using Regs = ChunkRegs<BITS, GLU>;
 
   MI_STAMP(0);
@@ -688,22 +693,28 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const size_t lds = small_lds_bytes(a.K, sk, tt, TTL, GLU ? 4 : 2);
   // with slabs a chunk's ring slot must not depend on the slab: the waves' K ranges have to start
   // at multiples of the ring depth
-  if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % MI_MOE_RING != 0) kw = 1;
+  const int by_lds0 = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
+  // two blocks per CU, 8-bit codes: eight chunks in flight (Mixtral shape -2..-4 %; with 4-bit codes, twice
+  // the unpacking and matrix work per byte, the same costs 8 % at 32 tokens of the Qwen3-235B shape)
+  const bool deep = BITS == 8 && (by_lds0 < (GLU ? 4 : 6) ? by_lds0 : (GLU ? 4 : 6)) <= 2;
+  if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % (deep ? MI_MOE_RING_DEEP : MI_MOE_RING) != 0) kw = 1;
   const int nw = 4 / kw;
   dim3 grid((unsigned)((a.N + 16 * nw - 1) / (16 * nw)), (unsigned)a.max_active);
   // blocks a CU holds: by LDS (160 KB) and by registers (4 with the gate/up kernel, 6 otherwise)
   const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
   const bool precise = (by_lds < (GLU ? 4 : 6) ? by_lds : (GLU ? 4 : 6)) <= MI_MOE_PRECISE_BELOW;
-#define MI_SMALL_LAUNCH(KWV, PR, SL, TGV)                                                        \
+#define MI_SMALL_LAUNCH(KWV, PR, SL, TGV, DV)                                                    \
   do {                                                                                         \
-    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV>), lds)) return; \
-    qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV><<<grid, 256, lds, st>>>(a, tt, sk);          \
+    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV>), lds)) return; \
+    qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV><<<grid, 256, lds, st>>>(a, tt, sk);      \
   } while (0)
 #define MI_SMALL(KWV, TGV)                                                                     \
   do {                                                                                         \
-    if (slabs) MI_SMALL_LAUNCH(KWV, true, true, TGV); /* long rows: few blocks per CU anyway */ \
-    else if (precise) MI_SMALL_LAUNCH(KWV, true, false, TGV);                                  \
-    else MI_SMALL_LAUNCH(KWV, false, false, TGV);                                              \
+    if (slabs && deep) MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING_DEEP);                \
+    else if (slabs) MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING); /* long rows: few blocks per CU anyway */ \
+    else if (precise && deep) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING_DEEP);        \
+    else if (precise) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING);                     \
+    else MI_SMALL_LAUNCH(KWV, false, false, TGV, MI_MOE_RING);                                 \
   } while (0)
   if constexpr (BITS == 4) {
     if (two_groups) {

@@ -697,6 +697,8 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // two blocks per CU, 8-bit codes: eight chunks in flight (Mixtral shape -2..-4 %; with 4-bit codes, twice
   // the unpacking and matrix work per byte, the same costs 8 % at 32 tokens of the Qwen3-235B shape)
   const bool deep = BITS == 8 && (by_lds0 < (GLU ? 4 : 6) ? by_lds0 : (GLU ? 4 : 6)) <= 2;
+  // one block per CU (one token of the Mixtral shape's down product: whole rows of 14336 values): sixteen
+  const bool deeper = deep && by_lds0 <= 1 && !slabs && ((chunks + kw - 1) / kw) % (2 * MI_MOE_RING_DEEP) == 0;
   if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % (deep ? MI_MOE_RING_DEEP : MI_MOE_RING) != 0) kw = 1;
   const int nw = 4 / kw;
   dim3 grid((unsigned)((a.N + 16 * nw - 1) / (16 * nw)), (unsigned)a.max_active);
@@ -712,6 +714,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   do {                                                                                         \
     if (slabs && deep) MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING_DEEP);                \
     else if (slabs) MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING); /* long rows: few blocks per CU anyway */ \
+    else if (precise && deeper) MI_SMALL_LAUNCH(KWV, true, false, TGV, 2 * MI_MOE_RING_DEEP);  \
     else if (precise && deep) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING_DEEP);        \
     else if (precise) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING);                     \
     else MI_SMALL_LAUNCH(KWV, false, false, TGV, MI_MOE_RING);                                 \

@@ -17,7 +17,9 @@ pytestmark = pytest.mark.gpu
 
 CASES = [
     # config, tokens, zipf s
+    ("qwen3_30b_a3b", 24, None),    # 1.5 rows per expert: short segments, five rows per pass and four blocks per CU
     ("qwen3_30b_a3b", 32, None),
+    ("qwen3_30b_a3b", 48, None),    # 3 rows per expert: eight rows per pass
     ("qwen3_30b_a3b", 160, None),   # 10 rows per expert: two token groups per pass, rows staged in slabs of 1024
     ("qwen3_30b_a3b", 200, 1.1),    # light batch, uneven routing: long segments tiled beside the streamed ones
     ("qwen3_30b_a3b", 4096, 1.1),
@@ -27,6 +29,7 @@ CASES = [
     ("mixtral_8x7b", 64, None),   # streamed, 16 rows per expert
     ("mixtral_8x7b", 96, None),   # 64-row tiles
     ("mixtral_8x7b", 2048, None),
+    ("qwen3_235b_a22b", 32, None),  # streamed, 4-bit rows of 4096 values (two blocks per CU)
     ("qwen3_235b_a22b", 8192, 1.3),
 ]
 

@@ -26,7 +26,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # what the same counters read for a plain copy kernel (profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt,
 # profiles/qmm_large_kernel_prefill_tokens4096_counters.txt);
 # counters cannot be read from inside this script, so the figure is carried here per workload.
-MEASURED_TRAFFIC_BYTES = {"decode": 2.056e8, "prefill": 5.50e8}
+MEASURED_TRAFFIC_BYTES = {"decode": 1.976e8, "prefill": 5.50e8}
 
 
 def parse():

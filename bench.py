@@ -226,7 +226,8 @@ def main():
         roofline = {"kernel": "qmm_small_kernel (gate/up + SwiGLU)", "bound": "hbm", "achieved": achieved,
                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                    "algorithmic_bytes_per_launch": head["gu_bytes"], **timing}
+                    "algorithmic_bytes_per_launch": head["gu_bytes"], **timing,
+                    "stream_probe": stream_probe(m, head["gu_bytes"], dev)}
     else:
         achieved = head["gu_flops"] / (kernel_ms * 1e-3) / 1e12
         roofline = {"kernel": "grouped qmm (gate/up + SwiGLU)", "bound": "mfma", "achieved": achieved,
@@ -251,6 +252,34 @@ def main():
         "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
     }
     print(json.dumps(out))
+
+
+def stream_probe(m, nbytes, dev):
+    """What a launch of the roofline kernel's size can pull from HBM on this box: the library's bare
+    streaming kernel (the product kernel's access shape, nothing else) over as many bytes as the
+    gate/up launch reads, launched back to back over 12 distinct regions (cold in every cache)."""
+    import torch
+    lib = m.capi.load_library()
+    size = max(32768, int(nbytes) // 32768 * 32768)
+    regions = 12
+    buf = torch.ones(regions * size, dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    def launch(i):
+        m.capi.check(lib.mi_moe_stream_probe(buf.data_ptr() + (i % regions) * size, size, sink.data_ptr(), st))
+    for i in range(regions):
+        launch(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 4 * regions
+    e0.record()
+    for i in range(reps):
+        launch(i)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / reps * 1e3
+    return {"bytes": size, "us_per_launch": us, "GBps": size / (us * 1e-6) / 1e9,
+            "frac_of_peak": size / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS}
 
 
 def cpu_baseline(cfg, block, T, seed, synth):

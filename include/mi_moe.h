@@ -206,6 +206,13 @@ int mi_moe_dequantize(const uint32_t *q, const uint16_t *scales, const uint16_t 
                       int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
                       float *w_hat, void *stream);
 
+/* ---- measurement aid; no counterpart in the reference.  A bare streaming kernel with the decode
+ * grouped product's access shape (a wave reads a 16 KiB tile from each half of buf, 64 bytes per row
+ * and instruction, four pieces in flight, four blocks per CU) over the first `bytes` bytes of buf
+ * (a multiple of 32768): what a launch of that size can pull from HBM.  bench.py reports it beside
+ * the roofline of the gate/up kernel.  sink: one device word (never written in practice). ---- */
+int mi_moe_stream_probe(const void *buf, size_t bytes, uint32_t *sink, void *stream);
+
 /* library version string, e.g. "mi_moe 0.1 gfx950" */
 const char *mi_moe_version(void);
 

@@ -20,7 +20,7 @@ EXPORTS = (
     "mi_moe_route", "mi_moe_dispatch_workspace_size", "mi_moe_dispatch",
     "mi_moe_gather_qmm_workspace_size", "mi_moe_gather_qmm",
     "mi_moe_quantized_matmul_workspace_size", "mi_moe_quantized_matmul", "mi_moe_swiglu", "mi_moe_combine",
-    "mi_moe_quantize", "mi_moe_dequantize",
+    "mi_moe_quantize", "mi_moe_dequantize", "mi_moe_stream_probe",
 )
 
 
@@ -100,6 +100,7 @@ def load_library():
         "mi_moe_combine": [vp, vp, vp, i64, i32, i32, vp, vp],
         "mi_moe_quantize": [vp, i64, i64, i32, i32, vp, vp, vp, vp],
         "mi_moe_dequantize": [vp, vp, vp, i64, i64, i32, i32, vp, vp],
+        "mi_moe_stream_probe": [vp, sz, vp, vp],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)

@@ -657,6 +657,16 @@ int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t 
   return 0;
 }
 
+int mi_moe_stream_probe(const void *buf, size_t bytes, uint32_t *sink, void *stream) {
+  if (bytes == 0) return 0;
+  if (bytes % 32768) return fail("stream_probe: bytes must be a multiple of 32768, got %zu", bytes);
+  if (bytes > ((size_t)1 << 34)) return fail("stream_probe: at most 16 GiB, got %zu", bytes);
+  if (!buf || !sink) return fail("stream_probe: buf and sink must be non-NULL");
+  if (reinterpret_cast<uintptr_t>(buf) % 16) return fail("stream_probe: buf must be 16-byte aligned");
+  MI_HIP(launch_stream_probe(buf, bytes, sink, static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
 int mi_moe_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm, int64_t T,
                    int32_t top_k, int32_t hidden, uint16_t *out, void *stream) {
   if (T < 0) return fail("combine: negative token count");

@@ -95,4 +95,49 @@ hipError_t launch_swiglu(const uint16_t *g, const uint16_t *u, int64_t n, uint16
   return hipGetLastError();
 }
 
+// Bare streaming kernel with the decode grouped product's access shape: a wave reads a 16 KiB tile
+// (16 rows of 1 KiB) from each of two arrays, 64 bytes per row and instruction, four pieces of
+// each in flight, and does nothing with them.  What a launch of a given size can pull from HBM.
+__global__ __launch_bounds__(256) void stream_probe_kernel(const uint32_t *__restrict__ p0,
+                                                           const uint32_t *__restrict__ p1,
+                                                           size_t n_tiles, uint32_t *sink) {
+  typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+  extern __shared__ unsigned char probe_lds[];
+  const int lane = threadIdx.x & 63;
+  const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (wave >= n_tiles) return;
+  const uint32_t voff = (lane & 15) * 1024 + (lane >> 4) * 16;
+  __amdgpu_buffer_rsrc_t r0 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p0 + wave * 4096), 0, 16384, 0x00020000);
+  __amdgpu_buffer_rsrc_t r1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p1 + wave * 4096), 0, 16384, 0x00020000);
+  constexpr int D = 4;
+  u32x4_t ring[D][2];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    ring[d][0] = __builtin_amdgcn_raw_buffer_load_b128(r0, voff, d * 64, 0);
+    ring[d][1] = __builtin_amdgcn_raw_buffer_load_b128(r1, voff, d * 64, 0);
+  }
+  uint32_t acc = 0;
+  for (int base = 0; base < 16; base += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const u32x4_t a = ring[d][0], b = ring[d][1];
+      acc += a[0] ^ a[1] ^ a[2] ^ a[3] ^ b[0] ^ b[1] ^ b[2] ^ b[3];
+      if (base + d + D < 16) {
+        ring[d][0] = __builtin_amdgcn_raw_buffer_load_b128(r0, voff, (base + d + D) * 64, 0);
+        ring[d][1] = __builtin_amdgcn_raw_buffer_load_b128(r1, voff, (base + d + D) * 64, 0);
+      }
+    }
+  }
+  if (acc == 0x12345678u) sink[0] = acc + probe_lds[0];  // keeps the loads alive; the buffer never holds such data
+}
+
+hipError_t launch_stream_probe(const void *buf, size_t bytes, uint32_t *sink, hipStream_t st) {
+  const size_t n_tiles = bytes / 32768;
+  if (n_tiles == 0) return hipSuccess;
+  const uint32_t *p0 = static_cast<const uint32_t *>(buf);
+  // 38000 bytes of LDS: four blocks per CU, as the product kernel at decode
+  stream_probe_kernel<<<(unsigned)((n_tiles + 3) / 4), 256, 38000, st>>>(p0, p0 + bytes / 8, n_tiles, sink);
+  return hipGetLastError();
+}
+
 }  // namespace mi_moe

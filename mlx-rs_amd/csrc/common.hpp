@@ -236,6 +236,7 @@ hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t
                                 hipStream_t st);
 hipError_t launch_swiglu(const uint16_t *g, const uint16_t *u, int64_t n, uint16_t *out,
                          hipStream_t st);
+hipError_t launch_stream_probe(const void *buf, size_t bytes, uint32_t *sink, hipStream_t st);
 hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm,
                           int64_t T, int k, int H, const uint16_t *residual, uint16_t *out,
                           hipStream_t st);

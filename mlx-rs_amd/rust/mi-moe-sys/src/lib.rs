@@ -89,5 +89,7 @@ extern "C" {
     pub fn mi_moe_quantize(w: *const f32, rows: i64, cols: i64, group_size: i32, bits: i32, q: *mut u32, scales: *mut u16, biases: *mut u16, stream: *mut c_void) -> c_int;
     pub fn mi_moe_dequantize(q: *const u32, scales: *const u16, biases: *const u16, rows: i64, cols: i64, group_size: i32, bits: i32, w_hat: *mut f32, stream: *mut c_void) -> c_int;
 
+    pub fn mi_moe_stream_probe(buf: *const c_void, bytes: usize, sink: *mut u32, stream: *mut c_void) -> c_int;
+
     pub fn mi_moe_version() -> *const c_char;
 }

@@ -84,6 +84,9 @@ def test_null_and_range_checks(lib):
     assert "bits" in m.capi.last_error()
     assert lib.mi_moe_combine(None, None, None, 4, 2, 64, None, None) != 0
     assert lib.mi_moe_swiglu(None, None, 8, None, None) != 0
+    assert lib.mi_moe_stream_probe(None, 1000, None, None) != 0
+    assert "32768" in m.capi.last_error()
+    assert lib.mi_moe_stream_probe(None, 32768, None, None) != 0
     assert lib.mi_moe_quantize(None, 2, 100, 64, 4, None, None, None, None) != 0
     assert "divisible" in m.capi.last_error()
     assert lib.mi_moe_dequantize(None, None, None, 2, 128, 64, 3, None, None) != 0
@@ -104,6 +107,7 @@ def test_null_and_range_checks(lib):
     assert "norm_weight" in m.capi.last_error()
     # empty inputs succeed without touching memory
     assert lib.mi_moe_swiglu(None, None, 0, None, None) == 0
+    assert lib.mi_moe_stream_probe(None, 0, None, None) == 0
     assert lib.mi_moe_combine(None, None, None, 0, 2, 64, None, None) == 0
 
 

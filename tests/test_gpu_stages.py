@@ -223,3 +223,19 @@ def test_untransposed_quantized_matmul_and_gather_qmm(orc, bits):
         refj = f32_of_bits(xs[lhs[j]]).astype(np.float64) @ orc.dequantize(W[rhs[j]], S[rhs[j]], B[rhs[j]], bits, 64).astype(np.float64)
         assert np.abs(yo[j] - refj).max() <= 1e-4
     assert_close_bf16(bits_u16(yg), orc.f32_to_bf16(yo), what="gather_qmm, transpose = false")
+
+
+def test_stream_probe_runs_and_rejects_bad_sizes():
+    """The measurement aid: a launch over a small buffer succeeds and leaves the sink alone;
+    sizes that are not whole 32 KiB tile pairs are refused with a message."""
+    import mlx_rs_amd as m
+    lib = m.capi.load_library()
+    buf = torch.ones(4 * 32768, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    m.capi.check(lib.mi_moe_stream_probe(buf.data_ptr(), 4 * 32768, sink.data_ptr(), st))
+    torch.cuda.synchronize()
+    assert int(sink.item()) == 0
+    assert lib.mi_moe_stream_probe(buf.data_ptr(), 1000, sink.data_ptr(), st) != 0
+    assert "32768" in m.capi.last_error()
+    assert lib.mi_moe_stream_probe(None, 32768, sink.data_ptr(), st) != 0

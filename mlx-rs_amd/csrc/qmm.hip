@@ -111,9 +111,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, ui
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
 
-template <int BITS, bool GLU>
+template <int BITS, bool TWO>
 struct ChunkRegs {
-  static constexpr int NM = GLU ? 2 : 1;
+  static constexpr int NM = TWO ? 2 : 1;
   u32x4_t q[NM];    // packed codes of this lane's weight row
 };
 
@@ -125,7 +125,7 @@ struct ChunkRegs {
 //                                 slabs the slab's sk/64 values of each of the 16 rows
 // xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
 __host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
-// Zeros that lanes without a token read.  Gate/up kernel (long rows, LDS decides how many blocks a
+// Zeros that lanes without a token read.  Gate/up kernel and paired tiles (long rows, LDS decides how many blocks a
 // CU holds): 64 bytes, read with a chunk stride of zero.  Down kernel: a whole zero row at the common
 // stride (the per-lane stride costs it 6 VGPRs, which would take it from 6 to 5 waves per SIMD).
 __host__ __device__ constexpr int zero_bytes(int sk, bool glu) { return glu ? 64 : 2 * sk + 16; }
@@ -153,16 +153,21 @@ __host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int 
 // of 9 to 16 rows then take one pass over the expert's weights instead of two.
 // D: chunks kept in flight per wave (ring depth).  Where a CU holds two blocks a wave may use 256
 // registers, and with 8-bit codes eight chunks in flight instead of four make up for the few waves.
-template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG, int D>
+// PAIR (plain products): a wave takes two adjacent row tiles (32 weight rows) against the same
+// activation operand, the way the gate/up kernel takes a gate and an up tile: half the blocks, each
+// with twice the weights to stream for one record read, one staging and one pair of barriers.
+template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG, int D, bool PAIR = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D > MI_MOE_RING ? 2 : 3, 8)))
 void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
+  static_assert(!PAIR || (!GLU && KW == 1 && !SLABS), "two row tiles per wave: plain product, whole rows, K not split");
+  constexpr bool TWO = GLU || PAIR;  // two weight tiles per chunk
   static_assert(TG == 1 || (TG == 2 && BITS == 4 && KW == 1), "two token groups: 4-bit, K not split over waves");
   constexpr int NW = 4 / KW;                    // row tiles per block
   constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one 16-byte load per lane)
   constexpr int XV = BITS == 4 ? 4 : 2;         // 16-byte pieces of activations per lane per chunk
-  constexpr int NM = GLU ? 2 : 1;
+  constexpr int NM = TWO ? 2 : 1;
   static_assert(D == MI_MOE_RING || PRECISE, "the deep ring goes with unconditional refills");
-  using Regs = ChunkRegs<BITS, GLU>;
+  using Regs = ChunkRegs<BITS, TWO>;
 
   MI_STAMP(0);
   // one 64-byte record says everything about this block's segment (uniform address: scalar loads)
@@ -181,7 +186,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   const int wk = wave % KW, wn = wave / KW;
   const int c = lane & 15, kb = lane >> 4;
   const int N = a.N, K = a.K;
-  const int n0 = (blockIdx.x * NW + wn) * 16;
+  const int n0 = (blockIdx.x * NW + wn) * (PAIR ? 32 : 16);
   const bool tile_ok = n0 < N;
   const int n = n0 + c;  // weight row of this lane (B operand / D column); rows >= N load zeros
 
@@ -202,6 +207,11 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     wr[1] = make_rsrc(a.w1 + ebase * (row_bytes / 4), (uint32_t)N * row_bytes);
     sr[1] = make_rsrc(a.s1 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
     br[1] = make_rsrc(a.b1 + ebase * groups_per_row, (uint32_t)N * groups_per_row * 2);
+  } else if constexpr (PAIR) {  // the same tensors, 16 rows further on
+    const uint32_t left = N > 16 ? (uint32_t)(N - 16) : 0u;
+    wr[1] = make_rsrc(a.w0 + (ebase + 16) * (row_bytes / 4), left * row_bytes);
+    sr[1] = make_rsrc(a.s0 + (ebase + 16) * groups_per_row, left * groups_per_row * 2);
+    br[1] = make_rsrc(a.b0 + (ebase + 16) * groups_per_row, left * groups_per_row * 2);
   }
   const uint32_t w_voff = (uint32_t)n * row_bytes + kb * 16;  // lane kb: 16 bytes of the 64-byte chunk
   // Long rows are staged a slab of sk K values at a time (sk = K: the whole row); the weight
@@ -270,8 +280,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
   extern __shared__ __align__(16) unsigned char lds[];
   unsigned char *lds_x = lds;
-  float *lds_gs = reinterpret_cast<float *>(lds + tt * xstride + zero_bytes(sk, GLU));  // [groups of the slab][TTL] sums of x
-  unsigned char *lds_sb = lds + tt * xstride + zero_bytes(sk, GLU) + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
+  float *lds_gs = reinterpret_cast<float *>(lds + tt * xstride + zero_bytes(sk, TWO));  // [groups of the slab][TTL] sums of x
+  unsigned char *lds_sb = lds + tt * xstride + zero_bytes(sk, TWO) + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
 
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait);
   // long rows in slabs: each slab brings its own piece (see the slab loop)
@@ -310,7 +320,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   __shared__ float red[KW > 1 ? KW : 1][KW > 1 ? NW : 1][NM][4][KW > 1 ? 64 : 1];
 
   // zero block and zero group sums (slots that carry no token stay zero for the whole launch)
-  for (int i = threadIdx.x; i < zero_bytes(sk, GLU) / 16; i += 256)
+  for (int i = threadIdx.x; i < zero_bytes(sk, TWO) / 16; i += 256)
     *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
   for (int i = threadIdx.x; i < groups_per_slab * TTL / 4; i += 256)
     *reinterpret_cast<uint4 *>(lds_gs + i * 4) = make_uint4(0, 0, 0, 0);
@@ -363,7 +373,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
         if (TG > 1 && g > 0) __builtin_amdgcn_sched_barrier(0);
         uint4 xv[XV];
 #pragma unroll
-        for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl[g] + (SLABS ? ch - slab_ch0 : ch) * (GLU ? xcs[g] : CH * 2) + i * 16);
+        for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl[g] + (SLABS ? ch - slab_ch0 : ch) * (TWO ? xcs[g] : CH * 2) + i * 16);
         f32x4_t acc[NM];
 #pragma unroll
         for (int m = 0; m < NM; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -477,7 +487,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
           const int ts_l = (BITS == 4 ? (c & 7) : c) + TT * g;
           bool a_on = ts_l < nt;
           if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
-          if constexpr (GLU) {
+          if constexpr (TWO) {
             xl[g] = a_on ? lds_x + ts_l * xstride + kb * (CH / 4) * 2 : lds_x + tt * xstride;
             xcs[g] = a_on ? CH * 2 : 0;
           } else {
@@ -610,6 +620,9 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
             int col = n;
             if (a.y_paired) col = (n & ~7) | ((n & 7) < 4 ? 2 * (n & 7) : 2 * ((n & 7) - 4) + 1);
             a.y[dst * N + col] = (uint16_t)(cvt_pk_bf16(v, 0.f) & 0xffffu);
+            if constexpr (PAIR) {  // the second tile: the same column 16 rows on (16 keeps the paired order)
+              if (n0 + 16 < N) a.y[dst * N + col + 16] = (uint16_t)(cvt_pk_bf16(res[g][1][r], 0.f) & 0xffffu);
+            }
           }
         }
     }
@@ -641,12 +654,18 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const bool two_groups = BITS == 4 && kw == 1 && longest > TT &&
                           a.total_rows >= (int64_t)MI_MOE_TG2_AVG * a.max_active;
   const int TTL = two_groups ? 2 * TT : TT;  // token slots of one pass
+  // plain products with two token groups per pass (five rows per expert and more): two row tiles per
+  // wave (measured: the down product of the 128-expert layer at 80 to 256 tokens -2..-4 us; with
+  // fewer rows per expert the same costs up to a microsecond: there more, smaller blocks win)
+  bool pair = !GLU && two_groups && a.K <= 2048 && a.N % 32 == 0;
+  const int n_tensors = (GLU || pair) ? 4 : 2;   // scale and bias tiles per wave in LDS
+  const int regs_blocks = (GLU || pair) ? 4 : 6;  // blocks a CU holds by registers
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
   int want = TTL;
   // short segments on average: stage fewer rows where the LDS saved buys a fourth block per CU (but
   // no fewer than that takes: a segment longer than the tile reads its expert's weights again)
   if (2 * a.total_rows <= MI_MOE_SHORT_AVG2 * (int64_t)a.max_active)
-    while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, GLU ? 4 : 2) > (size_t)160 * 1024) --want;
+    while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, n_tensors) > (size_t)160 * 1024) --want;
   if (longest < want) want = (int)longest;
   // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is
   // traded for occupancy only down to about twice the average segment; below that the tile keeps
@@ -658,8 +677,8 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int need = (int)(avg2 < 1 ? 1 : (avg2 < want ? avg2 : want));
   auto fit = [&](int slab) {
     int t = want;
-    while (t > need && small_lds_bytes(a.K, slab, t, TTL, GLU ? 4 : 2) > lds_soft) --t;
-    while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, GLU ? 4 : 2) > lds_hard) --t;
+    while (t > need && small_lds_bytes(a.K, slab, t, TTL, n_tensors) > lds_soft) --t;
+    while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, n_tensors) > lds_hard) --t;
     return t;
   };
   // The whole row, or the largest slab that does better, first in tokens per pass, then in blocks
@@ -670,7 +689,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // need rows of scales that are 16-byte aligned (K a multiple of 512).
   const int64_t launch_blocks = (int64_t)((a.N + 16 * (4 / kw) - 1) / (16 * (4 / kw))) * a.max_active;
   auto blocks_of = [&](int slab, int t) {
-    const int b = (int)((size_t)160 * 1024 / small_lds_bytes(a.K, slab, t, TTL, GLU ? 4 : 2));
+    const int b = (int)((size_t)160 * 1024 / small_lds_bytes(a.K, slab, t, TTL, n_tensors));
     const int cap = launch_blocks <= MI_MOE_CUS ? 1 : (2 * slab >= a.K ? 3 : 2);
     return b < cap ? b : cap;
   };
@@ -690,21 +709,23 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
     }
   }
   const bool slabs = sk < a.K;
-  const size_t lds = small_lds_bytes(a.K, sk, tt, TTL, GLU ? 4 : 2);
+  if (slabs) pair = false;  // (the sizes above then were on the safe side)
+  const size_t lds = small_lds_bytes(a.K, sk, tt, TTL, slabs ? (GLU ? 4 : 2) : n_tensors);
   // with slabs a chunk's ring slot must not depend on the slab: the waves' K ranges have to start
   // at multiples of the ring depth
   const int by_lds0 = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
   // two blocks per CU, 8-bit codes: eight chunks in flight (Mixtral shape -2..-4 %; with 4-bit codes, twice
   // the unpacking and matrix work per byte, the same costs 8 % at 32 tokens of the Qwen3-235B shape)
-  const bool deep = BITS == 8 && (by_lds0 < (GLU ? 4 : 6) ? by_lds0 : (GLU ? 4 : 6)) <= 2;
+  const bool deep = BITS == 8 && (by_lds0 < regs_blocks ? by_lds0 : regs_blocks) <= 2;
   // one block per CU (one token of the Mixtral shape's down product: whole rows of 14336 values): sixteen
   const bool deeper = deep && by_lds0 <= 1 && !slabs && ((chunks + kw - 1) / kw) % (2 * MI_MOE_RING_DEEP) == 0;
   if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % (deep ? MI_MOE_RING_DEEP : MI_MOE_RING) != 0) kw = 1;
   const int nw = 4 / kw;
-  dim3 grid((unsigned)((a.N + 16 * nw - 1) / (16 * nw)), (unsigned)a.max_active);
+  const int wave_rows = pair ? 32 : 16;  // weight rows per wave
+  dim3 grid((unsigned)((a.N + wave_rows * nw - 1) / (wave_rows * nw)), (unsigned)a.max_active);
   // blocks a CU holds: by LDS (160 KB) and by registers (4 with the gate/up kernel, 6 otherwise)
   const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
-  const bool precise = (by_lds < (GLU ? 4 : 6) ? by_lds : (GLU ? 4 : 6)) <= MI_MOE_PRECISE_BELOW;
+  const bool precise = (by_lds < regs_blocks ? by_lds : regs_blocks) <= MI_MOE_PRECISE_BELOW;
 #define MI_SMALL_LAUNCH(KWV, PR, SL, TGV, DV)                                                    \
   do {                                                                                         \
     if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV>), lds)) return; \
@@ -719,6 +740,27 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
     else if (precise) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING);                     \
     else MI_SMALL_LAUNCH(KWV, false, false, TGV, MI_MOE_RING);                                 \
   } while (0)
+  if constexpr (!GLU) {
+    if (pair) {  // (kw = 1, whole rows)
+#define MI_PAIR_LAUNCH(PR, TGV, DV)                                                              \
+  do {                                                                                         \
+    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, false, 1, PR, false, TGV, DV, true>), lds)) return; \
+    qmm_small_kernel<BITS, false, 1, PR, false, TGV, DV, true><<<grid, 256, lds, st>>>(a, tt, sk); \
+  } while (0)
+      if constexpr (BITS == 4) {
+        if (two_groups) {
+          if (precise) MI_PAIR_LAUNCH(true, 2, MI_MOE_RING);
+          else MI_PAIR_LAUNCH(false, 2, MI_MOE_RING);
+          return;
+        }
+      }
+      if (precise && deep) MI_PAIR_LAUNCH(true, 1, MI_MOE_RING_DEEP);
+      else if (precise) MI_PAIR_LAUNCH(true, 1, MI_MOE_RING);
+      else MI_PAIR_LAUNCH(false, 1, MI_MOE_RING);
+#undef MI_PAIR_LAUNCH
+      return;
+    }
+  }
   if constexpr (BITS == 4) {
     if (two_groups) {
       MI_SMALL(1, 2);

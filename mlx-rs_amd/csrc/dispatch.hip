@@ -39,26 +39,42 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(
   for (int i = tid; i < E; i += kDispThreads) blockhist[(int64_t)blockIdx.x * E + i] = lds[i];
 }
 
+// Per-block histograms -> counts, offsets, records, M tiles, and each block's first sorted position per
+// expert.  The blocks are dealt in G = 1024 / E' contiguous ranges (E' = E rounded up to a power of
+// two) to G threads per expert, so that a thread walks nb / G histograms, not nb.
 __global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
     uint32_t *__restrict__ blockhist, int nb, int E, uint32_t *__restrict__ counts,
     uint32_t *__restrict__ offsets, uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
     int cap256, uint32_t big_thr) {
   extern __shared__ uint32_t lds[];
   __shared__ uint32_t n_active;
-  uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E;
+  uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *part = lds + 3 * E;  // part[G][E]
   const int tid = threadIdx.x;
+  int ep = 1;
+  while (ep < E) ep <<= 1;
+  const int G = kDispThreads / ep;  // E <= 512: at least 2
+  const int e = tid % ep, g = tid / ep;
+  const int per = (nb + G - 1) / G;
+  const int b0 = g * per, b1 = b0 + per < nb ? b0 + per : nb;
+  if (e < E) {
+    uint32_t run = 0;
+    for (int b = b0; b < b1; ++b) run += blockhist[(int64_t)b * E + e];
+    part[g * E + e] = run;
+  }
+  __syncthreads();
   if (tid < E) {
     uint32_t run = 0;
-    for (int b = 0; b < nb; ++b) run += blockhist[(int64_t)b * E + tid];
+    for (int i = 0; i < G; ++i) run += part[i * E + tid];
     cnt[tid] = run;
   }
   __syncthreads();
   finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, cap256, big_thr, &n_active);
-  if (tid < E) {  // blockhist[b][e] <- first sorted position of expert e for block b
-    uint32_t run = cur[tid];
-    for (int b = 0; b < nb; ++b) {
-      uint32_t c = blockhist[(int64_t)b * E + tid];
-      blockhist[(int64_t)b * E + tid] = run;
+  if (e < E) {  // blockhist[b][e] <- first sorted position of expert e for block b
+    uint32_t run = cur[e];
+    for (int i = 0; i < g; ++i) run += part[i * E + e];
+    for (int b = b0; b < b1; ++b) {
+      uint32_t c = blockhist[(int64_t)b * E + e];
+      blockhist[(int64_t)b * E + e] = run;
       run += c;
     }
   }
@@ -102,7 +118,7 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
   uint32_t *blockhist = reinterpret_cast<uint32_t *>(scratch);
   const int nb = (int)((P + kSpan - 1) / kSpan);
   dispatch_hist_kernel<<<nb, kDispThreads, (size_t)E * 4, st>>>(flat, P, E, kSpan, blockhist);
-  dispatch_scan_kernel<<<1, kDispThreads, (size_t)3 * E * 4, st>>>(blockhist, nb, E, counts,
+  dispatch_scan_kernel<<<1, kDispThreads, ((size_t)3 * E + kDispThreads) * 4, st>>>(blockhist, nb, E, counts,
                                                                   offsets, work, mtiles, cap256, (uint32_t)big_thr);
   dispatch_scatter_kernel<<<nb, kDispThreads, (size_t)(1 + kDispWaves) * E * 4, st>>>(
       flat, P, E, nbits, k_div, kSpan, blockhist, perm, inv_perm, src_of);

@@ -85,7 +85,10 @@ extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
 #define MI_MOE_RING_DEEP 8  // chunks in flight per wave where a CU holds two blocks (registers are plentiful there)
 #endif
 #ifndef MI_MOE_TG2_AVG
-#define MI_MOE_TG2_AVG 5   // rows per active expert from which the 4-bit kernel takes two token groups per pass
+#define MI_MOE_TG2_AVG 6   // rows per active expert from which the 4-bit gate/up kernel takes two token groups per pass
+#endif
+#ifndef MI_MOE_TG2_AVG_PLAIN
+#define MI_MOE_TG2_AVG_PLAIN 8  // the same for plain products (short rows: a second pass costs them less)
 #endif
 #ifndef MI_MOE_CUS
 #define MI_MOE_CUS 256  // compute units of an MI355X
@@ -652,7 +655,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int64_t longest = a.max_streamed_rows > 0 && a.max_streamed_rows < a.max_rows_per_expert
                               ? a.max_streamed_rows : a.max_rows_per_expert;
   const bool two_groups = BITS == 4 && kw == 1 && longest > TT &&
-                          a.total_rows >= (int64_t)MI_MOE_TG2_AVG * a.max_active;
+                          a.total_rows >= (int64_t)(GLU ? MI_MOE_TG2_AVG : MI_MOE_TG2_AVG_PLAIN) * a.max_active;
   const int TTL = two_groups ? 2 * TT : TT;  // token slots of one pass
   // plain products with two token groups per pass (five rows per expert and more): two row tiles per
   // wave (measured: the down product of the 128-expert layer at 80 to 256 tokens -2..-4 us; with

@@ -657,7 +657,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const bool two_groups = BITS == 4 && kw == 1 && longest > TT &&
                           a.total_rows >= (int64_t)(GLU ? MI_MOE_TG2_AVG : MI_MOE_TG2_AVG_PLAIN) * a.max_active;
   const int TTL = two_groups ? 2 * TT : TT;  // token slots of one pass
-  // plain products with two token groups per pass (five rows per expert and more): two row tiles per
+  // plain products with two token groups per pass: two row tiles per
   // wave (measured: the down product of the 128-expert layer at 80 to 256 tokens -2..-4 us; with
   // fewer rows per expert the same costs up to a microsecond: there more, smaller blocks win)
   bool pair = !GLU && two_groups && a.K <= 2048 && a.N % 32 == 0;

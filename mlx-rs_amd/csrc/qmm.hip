@@ -137,10 +137,19 @@ __host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }
 // else) up to K = 4096; beyond, with slabs, the slab (a row of 14336 values has 7 KB of scales and
 // biases per wave and tensor: more than the activations of a few tokens)
 __host__ __device__ constexpr int sb_tile_k(int K, int sk) { return sk < K && K > 4096 ? sk : K; }
+// With K split over kw waves (whole rows staged) a wave parks the scales / biases of its own K range
+// only: K / kw values per row, when that range is a whole number of 16-byte pieces (512 values) of
+// 16-byte aligned rows of scales and its 16 rows fit two pieces per lane (the range <= 4096 values).
+// Returns that range, or 0: the whole row.
+__host__ __device__ constexpr int sb_range_k(int K, int kw, int bits) {
+  const int ch = bits == 4 ? 128 : 64, nchunks = K / ch, cpw = (nchunks + kw - 1) / kw;
+  return kw > 1 && K % 512 == 0 && (cpw * ch) % 512 == 0 && cpw * ch <= 4096 ? cpw * ch : 0;
+}
 // sk: K values of the activation rows staged at a time (a slab; the whole row when sk = K)
-__host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors) {
+// sbk: K values the scale / bias tiles cover when that is a wave's K range (sb_range_k), else 0
+__host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors, int sbk = 0) {
   return (size_t)tt * x_stride_bytes(sk) + zero_bytes(sk, n_tensors == 4) + (size_t)(sk / 64) * TT * 4 +
-         (size_t)4 * n_tensors * sb_tile_bytes(sb_tile_k(K, sk));
+         (size_t)4 * n_tensors * sb_tile_bytes(sbk > 0 && sk == K ? sbk : sb_tile_k(K, sk));
 }
 
 // PRECISE: the ring's refills are issued without a condition (chunk index clamped), so the compiler
@@ -221,8 +230,11 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   // stream, its ring and the accumulators run on across the slabs.
   const int sk = SLABS ? sk_arg : K;
   const int groups_per_slab = sk / 64;
-  const bool sb_whole = !SLABS || sb_tile_k(K, sk) == K;  // scale / bias tiles of the whole row, not per slab
-  const int sbt = sb_tile_bytes(sb_tile_k(K, sk));       // bytes of one tensor's scale (bias) tile in LDS
+  const int sb_rk = SLABS ? 0 : sb_range_k(K, KW, BITS);  // K split over the waves: the tiles of the wave's range
+  const bool sb_range = KW > 1 && sb_rk > 0;
+  const bool sb_whole = !sb_range && (!SLABS || sb_tile_k(K, sk) == K);  // scale / bias tiles of the whole row
+  const int sbt = sb_tile_bytes(sb_range ? sb_rk : sb_tile_k(K, sk));  // bytes of one tensor's scale (bias) tile in LDS
+  const int sb_groups = sb_range ? sb_rk / 64 : (sb_whole ? groups_per_row : groups_per_slab);  // per row in LDS
 
   // issue every global load of chunk ch into R
   auto issue = [&](int ch, Regs &R) {
@@ -268,7 +280,20 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   constexpr int SBI = 2;        // 16-byte loads per lane per tensor kept in registers (K <= 4096)
   const uint32_t sb_goff = (uint32_t)n0 * groups_per_row * 2 + lane * 16;
   u32x4_t sbv[NTEN][SBI];
-  if (sb_whole) {
+  if (KW > 1 && sb_range) {
+    // 16 rows x (range / 32) bytes in 16-byte pieces, piece p = row * ppr + piece of the row
+    const int ppr = sb_rk / 512;
+#pragma unroll
+    for (int t = 0; t < NTEN; ++t)
+#pragma unroll
+      for (int i = 0; i < SBI; ++i) {
+        const int p = i * 64 + lane;
+        if (p < 16 * ppr)
+          sbv[t][i] = __builtin_amdgcn_raw_buffer_load_b128(
+              (t & 1) ? br[t >> 1] : sr[t >> 1],
+              (uint32_t)(n0 + p / ppr) * groups_per_row * 2 + (uint32_t)(ch0 * CH / 64) * 2 + (p % ppr) * 16, 0, 0);
+      }
+  } else if (sb_whole) {
 #pragma unroll
     for (int t = 0; t < NTEN; ++t)
 #pragma unroll
@@ -289,7 +314,14 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait);
   // long rows in slabs: each slab brings its own piece (see the slab loop)
   auto park_sb = [&]() __attribute__((always_inline)) {
-  if (sb_whole) {
+  if (KW > 1 && sb_range) {
+#pragma unroll
+    for (int t = 0; t < NTEN; ++t)
+#pragma unroll
+      for (int i = 0; i < SBI; ++i)
+        if ((i * 64 + lane) * 16 < sbt)
+          *reinterpret_cast<u32x4_t *>(lds_sb + t * sbt + (i * 64 + lane) * 16) = sbv[t][i];
+  } else if (sb_whole) {
 #pragma unroll
     for (int t = 0; t < NTEN; ++t) {
 #pragma unroll
@@ -319,7 +351,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
       }
   };
   // this lane's scale / bias of the first chunk in LDS: row c, group (4-bit) kb >> 1 of the chunk's two
-  const unsigned char *sbl = lds_sb + (c * (sb_whole ? groups_per_row : groups_per_slab) + (BITS == 4 ? (kb >> 1) : 0)) * 2;
+  const unsigned char *sbl = lds_sb + (c * sb_groups + (BITS == 4 ? (kb >> 1) : 0)) * 2;
   __shared__ float red[KW > 1 ? KW : 1][KW > 1 ? NW : 1][NM][4][KW > 1 ? 64 : 1];
 
   // zero block and zero group sums (slots that carry no token stay zero for the whole launch)
@@ -419,7 +451,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
         const float4 xs = *reinterpret_cast<const float4 *>(gsl + (SLABS ? ch - slab_ch0 : ch) * (BITS == 4 ? 2 : 1) * TTL + TT * g);
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-          const int goff = (sb_whole ? ch : ch - slab_ch0) * (BITS == 4 ? 4 : 2);
+          const int goff = (sb_whole ? ch : (KW > 1 && sb_range ? ch - ch0 : ch - slab_ch0)) * (BITS == 4 ? 4 : 2);
           const float sc = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m) * sbt + goff));
           float bi = bf16_to_f32(*reinterpret_cast<const uint16_t *>(sbl + (2 * m + 1) * sbt + goff));
           if constexpr (BITS == 4) bi = __builtin_fmaf(-128.0f, sc, bi);
@@ -662,13 +694,14 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // fewer rows per expert the same costs up to a microsecond: there more, smaller blocks win)
   bool pair = !GLU && two_groups && a.K <= 2048 && a.N % 32 == 0;
   const int n_tensors = (GLU || pair) ? 4 : 2;   // scale and bias tiles per wave in LDS
+  const int sbk = sb_range_k(a.K, kw, BITS);     // K split over the waves: tiles of a wave's range only
   const int regs_blocks = (GLU || pair) ? 4 : 6;  // blocks a CU holds by registers
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
   int want = TTL;
   // short segments on average: stage fewer rows where the LDS saved buys a fourth block per CU (but
   // no fewer than that takes: a segment longer than the tile reads its expert's weights again)
   if (2 * a.total_rows <= MI_MOE_SHORT_AVG2 * (int64_t)a.max_active)
-    while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, n_tensors) > (size_t)160 * 1024) --want;
+    while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, n_tensors, sbk) > (size_t)160 * 1024) --want;
   if (longest < want) want = (int)longest;
   // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is
   // traded for occupancy only down to about twice the average segment; below that the tile keeps
@@ -680,8 +713,8 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int need = (int)(avg2 < 1 ? 1 : (avg2 < want ? avg2 : want));
   auto fit = [&](int slab) {
     int t = want;
-    while (t > need && small_lds_bytes(a.K, slab, t, TTL, n_tensors) > lds_soft) --t;
-    while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, n_tensors) > lds_hard) --t;
+    while (t > need && small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk) > lds_soft) --t;
+    while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk) > lds_hard) --t;
     return t;
   };
   // The whole row, or the largest slab that does better, first in tokens per pass, then in blocks
@@ -692,7 +725,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // need rows of scales that are 16-byte aligned (K a multiple of 512).
   const int64_t launch_blocks = (int64_t)((a.N + 16 * (4 / kw) - 1) / (16 * (4 / kw))) * a.max_active;
   auto blocks_of = [&](int slab, int t) {
-    const int b = (int)((size_t)160 * 1024 / small_lds_bytes(a.K, slab, t, TTL, n_tensors));
+    const int b = (int)((size_t)160 * 1024 / small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk));
     const int cap = launch_blocks <= MI_MOE_CUS ? 1 : (2 * slab >= a.K ? 3 : 2);
     return b < cap ? b : cap;
   };
@@ -713,7 +746,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   }
   const bool slabs = sk < a.K;
   if (slabs) pair = false;  // (the sizes above then were on the safe side)
-  const size_t lds = small_lds_bytes(a.K, sk, tt, TTL, slabs ? (GLU ? 4 : 2) : n_tensors);
+  const size_t lds = small_lds_bytes(a.K, sk, tt, TTL, slabs ? (GLU ? 4 : 2) : n_tensors, sbk);
   // with slabs a chunk's ring slot must not depend on the slab: the waves' K ranges have to start
   // at multiples of the ring depth
   const int by_lds0 = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));

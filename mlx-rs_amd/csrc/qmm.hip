@@ -128,7 +128,7 @@ struct ChunkRegs {
 //                                 slabs the slab's sk/64 values of each of the 16 rows
 // xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
 __host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
-// Zeros that lanes without a token read.  Gate/up kernel and paired tiles (long rows, LDS decides how many blocks a
+// Zeros that lanes without a token read.  Gate/up kernel, paired tiles, 8-bit codes with K split over the waves (long rows, LDS decides how many blocks a
 // CU holds): 64 bytes, read with a chunk stride of zero.  Down kernel: a whole zero row at the common
 // stride (the per-lane stride costs it 6 VGPRs, which would take it from 6 to 5 waves per SIMD).
 __host__ __device__ constexpr int zero_bytes(int sk, bool glu) { return glu ? 64 : 2 * sk + 16; }
@@ -139,16 +139,18 @@ __host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }
 __host__ __device__ constexpr int sb_tile_k(int K, int sk) { return sk < K && K > 4096 ? sk : K; }
 // With K split over kw waves (whole rows staged) a wave parks the scales / biases of its own K range
 // only: K / kw values per row, when that range is a whole number of 16-byte pieces (512 values) of
-// 16-byte aligned rows of scales and its 16 rows fit two pieces per lane (the range <= 4096 values).
+// 16-byte aligned rows of scales and its 16 rows fit the pieces a lane holds (two with 4-bit codes: the range
+// <= 4096 values; four with 8-bit codes: <= 8192).
 // Returns that range, or 0: the whole row.
 __host__ __device__ constexpr int sb_range_k(int K, int kw, int bits) {
   const int ch = bits == 4 ? 128 : 64, nchunks = K / ch, cpw = (nchunks + kw - 1) / kw;
-  return kw > 1 && K % 512 == 0 && (cpw * ch) % 512 == 0 && cpw * ch <= 4096 ? cpw * ch : 0;
+  return kw > 1 && K % 512 == 0 && (cpw * ch) % 512 == 0 && cpw * ch <= (bits == 8 ? 8192 : 4096) ? cpw * ch : 0;
 }
 // sk: K values of the activation rows staged at a time (a slab; the whole row when sk = K)
 // sbk: K values the scale / bias tiles cover when that is a wave's K range (sb_range_k), else 0
-__host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors, int sbk = 0) {
-  return (size_t)tt * x_stride_bytes(sk) + zero_bytes(sk, n_tensors == 4) + (size_t)(sk / 64) * TT * 4 +
+// zb: the 64-byte block of zeros (gate/up, paired tiles, K split over the waves), not a zero row
+__host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors, int sbk, bool zb) {
+  return (size_t)tt * x_stride_bytes(sk) + zero_bytes(sk, zb) + (size_t)(sk / 64) * TT * 4 +
          (size_t)4 * n_tensors * sb_tile_bytes(sbk > 0 && sk == K ? sbk : sb_tile_k(K, sk));
 }
 
@@ -173,6 +175,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D > MI_MOE_
 void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   static_assert(!PAIR || (!GLU && KW == 1 && !SLABS), "two row tiles per wave: plain product, whole rows, K not split");
   constexpr bool TWO = GLU || PAIR;  // two weight tiles per chunk
+  // lanes without a token read a 64-byte block of zeros (see zero_bytes); with 4-bit codes and K split over
+  // the waves (a few tokens of a 128-expert layer) the plain kernel keeps its zero row: the block costs it
+  // registers and a quarter of a microsecond there
+  constexpr bool ZB = TWO || (KW > 1 && BITS == 8);
   static_assert(TG == 1 || (TG == 2 && BITS == 4 && KW == 1), "two token groups: 4-bit, K not split over waves");
   constexpr int NW = 4 / KW;                    // row tiles per block
   constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one 16-byte load per lane)
@@ -277,7 +283,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   // scales and biases of the wave's 16 rows: K/2 contiguous bytes per tensor, fetched with
   // fully coalesced 16-byte loads now and parked in LDS (wave-private) before the chunk loop
   constexpr int NTEN = 2 * NM;  // tensors: scales, biases (x gate, up)
-  constexpr int SBI = 2;        // 16-byte loads per lane per tensor kept in registers (K <= 4096)
+  constexpr int SBI = KW > 1 && BITS == 8 ? 4 : 2;  // 16-byte loads per lane per tensor kept in registers
   const uint32_t sb_goff = (uint32_t)n0 * groups_per_row * 2 + lane * 16;
   u32x4_t sbv[NTEN][SBI];
   if (KW > 1 && sb_range) {
@@ -308,8 +314,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
   extern __shared__ __align__(16) unsigned char lds[];
   unsigned char *lds_x = lds;
-  float *lds_gs = reinterpret_cast<float *>(lds + tt * xstride + zero_bytes(sk, TWO));  // [groups of the slab][TTL] sums of x
-  unsigned char *lds_sb = lds + tt * xstride + zero_bytes(sk, TWO) + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
+  float *lds_gs = reinterpret_cast<float *>(lds + tt * xstride + zero_bytes(sk, ZB));  // [groups of the slab][TTL] sums of x
+  unsigned char *lds_sb = lds + tt * xstride + zero_bytes(sk, ZB) + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
 
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait);
   // long rows in slabs: each slab brings its own piece (see the slab loop)
@@ -355,7 +361,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   __shared__ float red[KW > 1 ? KW : 1][KW > 1 ? NW : 1][NM][4][KW > 1 ? 64 : 1];
 
   // zero block and zero group sums (slots that carry no token stay zero for the whole launch)
-  for (int i = threadIdx.x; i < zero_bytes(sk, TWO) / 16; i += 256)
+  for (int i = threadIdx.x; i < zero_bytes(sk, ZB) / 16; i += 256)
     *reinterpret_cast<uint4 *>(lds_x + tt * xstride + i * 16) = make_uint4(0, 0, 0, 0);
   for (int i = threadIdx.x; i < groups_per_slab * TTL / 4; i += 256)
     *reinterpret_cast<uint4 *>(lds_gs + i * 4) = make_uint4(0, 0, 0, 0);
@@ -408,7 +414,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
         if (TG > 1 && g > 0) __builtin_amdgcn_sched_barrier(0);
         uint4 xv[XV];
 #pragma unroll
-        for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl[g] + (SLABS ? ch - slab_ch0 : ch) * (TWO ? xcs[g] : CH * 2) + i * 16);
+        for (int i = 0; i < XV; ++i) xv[i] = *reinterpret_cast<const uint4 *>(xl[g] + (SLABS ? ch - slab_ch0 : ch) * (ZB ? xcs[g] : CH * 2) + i * 16);
         f32x4_t acc[NM];
 #pragma unroll
         for (int m = 0; m < NM; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -522,7 +528,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
           const int ts_l = (BITS == 4 ? (c & 7) : c) + TT * g;
           bool a_on = ts_l < nt;
           if constexpr (BITS == 4) a_on = a_on && ((kb >> 1) == (c >> 3));
-          if constexpr (TWO) {
+          if constexpr (ZB) {
             xl[g] = a_on ? lds_x + ts_l * xstride + kb * (CH / 4) * 2 : lds_x + tt * xstride;
             xcs[g] = a_on ? CH * 2 : 0;
           } else {
@@ -695,13 +701,14 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   bool pair = !GLU && two_groups && a.K <= 2048 && a.N % 32 == 0;
   const int n_tensors = (GLU || pair) ? 4 : 2;   // scale and bias tiles per wave in LDS
   const int sbk = sb_range_k(a.K, kw, BITS);     // K split over the waves: tiles of a wave's range only
+  const bool zb = GLU || pair || (kw > 1 && BITS == 8);  // a block of zeros instead of a zero row (see zero_bytes)
   const int regs_blocks = (GLU || pair) ? 4 : 6;  // blocks a CU holds by registers
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
   int want = TTL;
   // short segments on average: stage fewer rows where the LDS saved buys a fourth block per CU (but
   // no fewer than that takes: a segment longer than the tile reads its expert's weights again)
   if (2 * a.total_rows <= MI_MOE_SHORT_AVG2 * (int64_t)a.max_active)
-    while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, n_tensors, sbk) > (size_t)160 * 1024) --want;
+    while (want > MI_MOE_SHORT_TT && 4 * small_lds_bytes(a.K, a.K, want, TTL, n_tensors, sbk, zb) > (size_t)160 * 1024) --want;
   if (longest < want) want = (int)longest;
   // Every token of a segment beyond tt costs another pass over the expert's weights, so LDS is
   // traded for occupancy only down to about twice the average segment; below that the tile keeps
@@ -713,8 +720,8 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int need = (int)(avg2 < 1 ? 1 : (avg2 < want ? avg2 : want));
   auto fit = [&](int slab) {
     int t = want;
-    while (t > need && small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk) > lds_soft) --t;
-    while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk) > lds_hard) --t;
+    while (t > need && small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk, zb) > lds_soft) --t;
+    while (t > 1 && small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk, zb) > lds_hard) --t;
     return t;
   };
   // The whole row, or the largest slab that does better, first in tokens per pass, then in blocks
@@ -725,7 +732,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // need rows of scales that are 16-byte aligned (K a multiple of 512).
   const int64_t launch_blocks = (int64_t)((a.N + 16 * (4 / kw) - 1) / (16 * (4 / kw))) * a.max_active;
   auto blocks_of = [&](int slab, int t) {
-    const int b = (int)((size_t)160 * 1024 / small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk));
+    const int b = (int)((size_t)160 * 1024 / small_lds_bytes(a.K, slab, t, TTL, n_tensors, sbk, zb));
     const int cap = launch_blocks <= MI_MOE_CUS ? 1 : (2 * slab >= a.K ? 3 : 2);
     return b < cap ? b : cap;
   };
@@ -746,7 +753,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   }
   const bool slabs = sk < a.K;
   if (slabs) pair = false;  // (the sizes above then were on the safe side)
-  const size_t lds = small_lds_bytes(a.K, sk, tt, TTL, slabs ? (GLU ? 4 : 2) : n_tensors, sbk);
+  size_t lds = small_lds_bytes(a.K, sk, tt, TTL, slabs ? (GLU ? 4 : 2) : n_tensors, sbk, zb);
   // with slabs a chunk's ring slot must not depend on the slab: the waves' K ranges have to start
   // at multiples of the ring depth
   const int by_lds0 = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
@@ -754,8 +761,13 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // the unpacking and matrix work per byte, the same costs 8 % at 32 tokens of the Qwen3-235B shape)
   const bool deep = BITS == 8 && (by_lds0 < regs_blocks ? by_lds0 : regs_blocks) <= 2;
   // one block per CU (one token of the Mixtral shape's down product: whole rows of 14336 values): sixteen
-  const bool deeper = deep && by_lds0 <= 1 && !slabs && ((chunks + kw - 1) / kw) % (2 * MI_MOE_RING_DEEP) == 0;
-  if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % (deep ? MI_MOE_RING_DEEP : MI_MOE_RING) != 0) kw = 1;
+  const int64_t grid_blocks = (int64_t)((a.N + 16 * (4 / kw) - 1) / (16 * (4 / kw))) * a.max_active;
+  const bool deeper = deep && (by_lds0 <= 1 || grid_blocks <= MI_MOE_CUS) && !slabs &&
+                      ((chunks + kw - 1) / kw) % (2 * MI_MOE_RING_DEEP) == 0;
+  if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % (deep ? MI_MOE_RING_DEEP : MI_MOE_RING) != 0) {
+    kw = 1;  // (and with it the zero row instead of the block of zeros)
+    lds = small_lds_bytes(a.K, sk, tt, TTL, GLU ? 4 : 2, 0, GLU);
+  }
   const int nw = 4 / kw;
   const int wave_rows = pair ? 32 : 16;  // weight rows per wave
   dim3 grid((unsigned)((a.N + wave_rows * nw - 1) / (wave_rows * nw)), (unsigned)a.max_active);

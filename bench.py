@@ -24,9 +24,10 @@ HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # HBM bytes per launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE scaled by
 # what the same counters read for a plain copy kernel (profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt,
+# profiles/qmm_small_kernel_decode_mixtral_batch1.txt,
 # profiles/qmm_large_kernel_prefill_tokens4096_counters.txt);
 # counters cannot be read from inside this script, so the figure is carried here per workload.
-MEASURED_TRAFFIC_BYTES = {"decode": 1.976e8, "prefill": 5.50e8}
+MEASURED_TRAFFIC_BYTES = {"decode": 1.976e8, "prefill": 5.50e8, "mixtral_decode": 2.530e8}
 
 
 def parse():

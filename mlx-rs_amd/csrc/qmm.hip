@@ -125,12 +125,14 @@ struct ChunkRegs {
 //   then groups x TT fp32         sum of x over each quantisation group, per token slot
 //   then per wave, per tensor     the bf16 scales (and biases) of the wave's 16 weight rows: a flat
 //                                 copy of 16 * K/64 values (they are contiguous in memory), or with
-//                                 slabs the slab's sk/64 values of each of the 16 rows
+//                                 slabs the slab's sk/64 values of each of the 16 rows, or with K split
+//                                 over the waves the values of the wave's K range (sb_range_k)
 // xstride carries 16 bytes of padding so that token slots spread over the LDS banks.
 __host__ __device__ constexpr int x_stride_bytes(int K) { return 2 * K + 16; }
-// Zeros that lanes without a token read.  Gate/up kernel, paired tiles, 8-bit codes with K split over the waves (long rows, LDS decides how many blocks a
-// CU holds): 64 bytes, read with a chunk stride of zero.  Down kernel: a whole zero row at the common
-// stride (the per-lane stride costs it 6 VGPRs, which would take it from 6 to 5 waves per SIMD).
+// Zeros that lanes without a token read.  Gate/up kernel, paired tiles, 8-bit codes with K split over
+// the waves (long rows, LDS decides how many blocks a CU holds): 64 bytes, read with a chunk stride of
+// zero.  Plain products otherwise: a whole zero row at the common stride (the per-lane stride costs
+// them 6 VGPRs, which would take the down kernel from 6 to 5 waves per SIMD).
 __host__ __device__ constexpr int zero_bytes(int sk, bool glu) { return glu ? 64 : 2 * sk + 16; }
 __host__ __device__ constexpr int sb_tile_bytes(int K) { return 32 * (K / 64); }  // 16 rows x K/64 bf16
 // K values the scale / bias tiles in LDS cover: the whole row (fetched once, ahead of everything
@@ -148,7 +150,7 @@ __host__ __device__ constexpr int sb_range_k(int K, int kw, int bits) {
 }
 // sk: K values of the activation rows staged at a time (a slab; the whole row when sk = K)
 // sbk: K values the scale / bias tiles cover when that is a wave's K range (sb_range_k), else 0
-// zb: the 64-byte block of zeros (gate/up, paired tiles, K split over the waves), not a zero row
+// zb: the 64-byte block of zeros, not a zero row (see zero_bytes)
 __host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int TT, int n_tensors, int sbk, bool zb) {
   return (size_t)tt * x_stride_bytes(sk) + zero_bytes(sk, zb) + (size_t)(sk / 64) * TT * 4 +
          (size_t)4 * n_tensors * sb_tile_bytes(sbk > 0 && sk == K ? sbk : sb_tile_k(K, sk));

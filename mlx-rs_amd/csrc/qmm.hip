@@ -688,7 +688,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int chunks = a.K / (BITS == 4 ? 128 : 64);
   int kw = 1;  // measured on the 128-expert layer: 2 pays below ~2000 row tiles, 4 only when nearly empty
   if (tiles < 256 && chunks >= 8) kw = 4;
-  else if (tiles < 2048 && chunks >= 4) kw = 2;
+  else if (tiles < (GLU ? 2048 : 1024) && chunks >= 4) kw = 2;  // (plain products: one token of the 128-expert layer is 1024 tiles, -0.5 us unsplit)
   // 4-bit, segments that can be longer than one MFMA tile's 8 tokens, and long enough on average
   // for it to matter: two token groups per pass (a 9- to 16-row segment then reads its expert's
   // weights once, not twice)

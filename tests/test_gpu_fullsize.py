@@ -17,6 +17,8 @@ pytestmark = pytest.mark.gpu
 
 CASES = [
     # config, tokens, zipf s
+    ("qwen3_30b_a3b", 1, None),     # K split over the waves: scale/bias tiles of a wave's K range
+    ("qwen3_30b_a3b", 4, None),
     ("qwen3_30b_a3b", 24, None),    # 1.5 rows per expert: short segments, five rows per pass and four blocks per CU
     ("qwen3_30b_a3b", 32, None),
     ("qwen3_30b_a3b", 48, None),    # 3 rows per expert: eight rows per pass
@@ -29,6 +31,7 @@ CASES = [
     ("mixtral_8x7b", 64, None),   # streamed, 16 rows per expert
     ("mixtral_8x7b", 96, None),   # 64-row tiles
     ("mixtral_8x7b", 2048, None),
+    ("qwen3_235b_a22b", 2, None),   # K split over the waves, rows of 4096 4-bit values
     ("qwen3_235b_a22b", 32, None),  # streamed, 4-bit rows of 4096 values (two blocks per CU)
     ("qwen3_235b_a22b", 8192, 1.3),
 ]

@@ -5,6 +5,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <exception>
+#include <memory>
+#include <mutex>
 #include <new>
 
 #include "common.hpp"
@@ -15,9 +18,20 @@ using namespace mi_moe;
 namespace {
 
 thread_local char g_last_error[512] = "";
-void (*g_handler)(const char *, void *) = nullptr;
-void *g_handler_data = nullptr;
-void (*g_handler_dtor)(void *) = nullptr;
+
+// The registered handler with its data.  A failing thread takes a reference under the lock and calls
+// the handler outside it, so a handler swapped meanwhile stays alive (its dtor runs when the last
+// reference goes) and a handler may itself register another one.
+struct Handler {
+  void (*fn)(const char *, void *);
+  void *data;
+  void (*dtor)(void *);
+  ~Handler() {
+    if (dtor && data) dtor(data);
+  }
+};
+std::mutex g_handler_lock;
+std::shared_ptr<Handler> g_handler;
 
 int fail(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 int fail(const char *fmt, ...) {
@@ -25,9 +39,19 @@ int fail(const char *fmt, ...) {
   va_start(ap, fmt);
   vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
   va_end(ap);
-  if (g_handler) g_handler(g_last_error, g_handler_data);
+  std::shared_ptr<Handler> h;
+  {
+    std::lock_guard<std::mutex> g(g_handler_lock);
+    h = g_handler;
+  }
+  if (h && h->fn) h->fn(g_last_error, h->data);
   return 1;
 }
+
+// No exception leaves an entry point: every extern "C" body is a function-try-block that ends in this.
+#define MI_CATCH(name)                                                                  \
+  catch (const std::exception &ex_) { return fail(name ": %s", ex_.what()); }           \
+  catch (...) { return fail(name ": unknown C++ exception"); }
 
 int hip_fail(const char *what, hipError_t e) {
   return fail("%s: %s", what, hipGetErrorString(e));
@@ -67,11 +91,13 @@ int check_qmat(const mi_moe_qmat &m, const char *name) {
   return 0;
 }
 
-// carve consecutive 256-byte aligned regions out of a workspace
+// carve consecutive 256-byte aligned regions out of a workspace; the first one starts at the next
+// 256-byte boundary (every *_workspace_size reserves 256 bytes for that)
 struct Carver {
   char *base;
   size_t off = 0;
-  explicit Carver(void *p) : base(static_cast<char *>(p)) {}
+  explicit Carver(void *p)
+      : base(reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(p) + 255u) & ~(uintptr_t)255u)) {}
   template <typename T>
   T *take(size_t n) {
     T *p = reinterpret_cast<T *>(base + off);
@@ -156,16 +182,22 @@ extern "C" {
 const char *mi_moe_last_error(void) { return g_last_error; }
 
 void mi_moe_set_error_handler(void (*handler)(const char *, void *), void *data,
-                              void (*dtor)(void *)) {
-  if (g_handler_dtor && g_handler_data) g_handler_dtor(g_handler_data);
-  g_handler = handler;
-  g_handler_data = data;
-  g_handler_dtor = dtor;
+                              void (*dtor)(void *)) try {
+  std::shared_ptr<Handler> next, old;
+  if (handler || data || dtor) next = std::make_shared<Handler>(Handler{handler, data, dtor});
+  {
+    std::lock_guard<std::mutex> g(g_handler_lock);
+    old = std::move(g_handler);
+    g_handler = std::move(next);
+  }
+  // `old` goes here, outside the lock: its dtor runs once no failing thread still uses it
+} catch (...) {
+  // out of host memory: the previous handler stays
 }
 
 const char *mi_moe_version(void) { return "mi_moe 0.1 gfx950"; }
 
-int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_moe_handle *out) {
+int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_moe_handle *out) try {
   if (!out) return fail("create: out handle is NULL");
   if (check_config(cfg)) return 1;
   if (!weights) return fail("create: weights is NULL");
@@ -194,21 +226,21 @@ int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_mo
   }
   *out = h;
   return 0;
-}
+} MI_CATCH("create")
 
-int mi_moe_destroy(mi_moe_handle h) {
+int mi_moe_destroy(mi_moe_handle h) try {
   destroy_handle(h);
   return 0;
-}
+} MI_CATCH("destroy")
 
-int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *bytes) {
+int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *bytes) try {
   if (!bytes) return fail("workspace_size: bytes is NULL");
   if (check_config(cfg)) return 1;
   if (max_tokens < 0) return fail("workspace_size: negative token count");
   if (max_tokens * cfg->top_k > (int64_t)1 << 30) return fail("workspace_size: too many (token, expert) pairs");
   *bytes = carve_forward(*cfg, max_tokens, nullptr).bytes + 256;
   return 0;
-}
+} MI_CATCH("workspace_size")
 
 // The launch sequence of one forward.  ev: nullptr, or kStages + 1 events recorded on the
 // stream before the first launch and after each stage.
@@ -397,22 +429,22 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
 }
 
 int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
-                   size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream) {
+                   size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream) try {
   return forward_impl(h, x, T, out, workspace, workspace_bytes, dbg, static_cast<hipStream_t>(stream), nullptr);
-}
+} MI_CATCH("forward")
 
 int mi_moe_forward_residual(mi_moe_handle h, const uint16_t *x, const uint16_t *norm_weight, float eps,
                             int64_t T, uint16_t *out, void *workspace, size_t workspace_bytes,
-                            const mi_moe_debug_out *dbg, void *stream) {
+                            const mi_moe_debug_out *dbg, void *stream) try {
   if (!norm_weight || !aligned16(norm_weight)) return fail("forward_residual: norm_weight must be non-NULL and 16-byte aligned");
   if (!(eps >= 0.f)) return fail("forward_residual: eps must be non-negative");
   if (x == out) return fail("forward_residual: out must not alias x (x is read again at the end)");
   return forward_impl(h, x, T, out, workspace, workspace_bytes, dbg, static_cast<hipStream_t>(stream), nullptr,
                       norm_weight, eps);
-}
+} MI_CATCH("forward_residual")
 
 int mi_moe_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int32_t hidden,
-                    uint16_t *out, void *stream) {
+                    uint16_t *out, void *stream) try {
   if (T < 0) return fail("rms_norm: negative row count");
   if (hidden <= 0 || hidden % 8) return fail("rms_norm: hidden must be a positive multiple of 8, got %d", hidden);
   if (!(eps >= 0.f)) return fail("rms_norm: eps must be non-negative");
@@ -421,14 +453,20 @@ int mi_moe_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_
   if (!aligned16(x) || !aligned16(weight) || !aligned16(out)) return fail("rms_norm: pointers must be 16-byte aligned");
   MI_HIP(launch_rms_norm(x, weight, eps, T, hidden, out, static_cast<hipStream_t>(stream)));
   return 0;
-}
+} MI_CATCH("rms_norm")
 
 int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
-                         size_t workspace_bytes, void *stream, float *stage_ms) {
+                         size_t workspace_bytes, void *stream, float *stage_ms) try {
   if (!stage_ms) return fail("forward_timed: stage_ms is NULL");
   hipStream_t st = static_cast<hipStream_t>(stream);
   hipEvent_t ev[MI_MOE_N_STAGES + 1];
-  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) MI_HIP(hipEventCreate(&ev[i]));
+  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) {
+    const hipError_t e = hipEventCreate(&ev[i]);
+    if (e != hipSuccess) {
+      while (--i >= 0) (void)hipEventDestroy(ev[i]);
+      return hip_fail("hipEventCreate", e);
+    }
+  }
   int rc = forward_impl(h, x, T, out, workspace, workspace_bytes, nullptr, st, ev);
   if (rc == 0 && T > 0) {
     hipError_t e = hipEventSynchronize(ev[MI_MOE_N_STAGES]);
@@ -440,21 +478,21 @@ int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t
   }
   for (int i = 0; i <= MI_MOE_N_STAGES; ++i) (void)hipEventDestroy(ev[i]);
   return rc;
-}
+} MI_CATCH("forward_timed")
 
 // ------------------------------------------------------------------ stage level
 
-int mi_moe_route_workspace_size(int32_t n_experts, int64_t T, size_t *bytes) {
+int mi_moe_route_workspace_size(int32_t n_experts, int64_t T, size_t *bytes) try {
   if (!bytes) return fail("route_workspace_size: bytes is NULL");
   if (n_experts < 1 || n_experts > 512 || T < 0) return fail("route_workspace_size: bad arguments");
   *bytes = align_up((size_t)T * n_experts * 2) + 256;
   return 0;
-}
+} MI_CATCH("route_workspace_size")
 
 int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *router_bias, int64_t T,
                  int32_t hidden, int32_t n_experts, int32_t top_k, int32_t score_mode,
                  uint32_t *topk_idx, uint16_t *topk_w, uint16_t *logits_out, void *workspace,
-                 size_t workspace_bytes, void *stream) {
+                 size_t workspace_bytes, void *stream) try {
   if (T < 0) return fail("route: negative token count");
   if (hidden <= 0 || hidden % 64) return fail("route: hidden must be a positive multiple of 64, got %d", hidden);
   if (n_experts < 1 || n_experts > 512) return fail("route: n_experts must be in [1, 512], got %d", n_experts);
@@ -474,19 +512,19 @@ int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *route
   MI_HIP(launch_router_logits(x, router_w, router_bias, T, hidden, n_experts, logits, st));
   MI_HIP(launch_router_select(logits, T, n_experts, top_k, score_mode, topk_idx, topk_w, st));
   return 0;
-}
+} MI_CATCH("route")
 
-int mi_moe_dispatch_workspace_size(int32_t n_experts, int64_t P, size_t *bytes) {
+int mi_moe_dispatch_workspace_size(int32_t n_experts, int64_t P, size_t *bytes) try {
   if (!bytes) return fail("dispatch_workspace_size: bytes is NULL");
   if (n_experts < 1 || n_experts > 512 || P < 0) return fail("dispatch_workspace_size: bad arguments");
   // scratch + counts/offsets/active/n_active stand-ins for outputs the caller leaves NULL
   *bytes = align_up(dispatch_workspace_bytes(n_experts, P)) + 256;
   return 0;
-}
+} MI_CATCH("dispatch_workspace_size")
 
 int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts, uint32_t *counts,
                     uint32_t *offsets, uint32_t *perm, uint32_t *inv_perm, void *workspace,
-                    size_t workspace_bytes, void *stream) {
+                    size_t workspace_bytes, void *stream) try {
   if (P < 0 || P > (int64_t)1 << 30) return fail("dispatch: pair count out of range");
   if (n_experts < 1 || n_experts > 512) return fail("dispatch: n_experts must be in [1, 512], got %d", n_experts);
   if (!perm) return fail("dispatch: perm must be non-NULL");
@@ -500,22 +538,22 @@ int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts
   MI_HIP(launch_dispatch(expert_of_pair, P, n_experts, 1, counts, offsets, perm, inv_perm, nullptr, nullptr,
                          nullptr, 0, 0, scratch, st));
   return 0;
-}
+} MI_CATCH("dispatch")
 
-int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M, size_t *bytes) {
+int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M, size_t *bytes) try {
   if (!bytes) return fail("gather_qmm_workspace_size: bytes is NULL");
   if (n_experts < 1 || n_experts > 512 || n_idx < 0 || M < 1) return fail("gather_qmm_workspace_size: bad arguments");
   const int64_t rows = n_idx * M;  // perm and the (src, dst) row maps hold one entry per output row
   *bytes = align_up(dispatch_workspace_bytes(n_experts, rows)) + 2 * align_up((size_t)(n_experts + 1) * 4) +
            align_up((size_t)n_experts * 64) + 3 * align_up((size_t)rows * 4) + 256;
   return 0;
-}
+} MI_CATCH("gather_qmm_workspace_size")
 
 int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
                       const uint16_t *biases, const uint32_t *lhs_indices, const uint32_t *rhs_indices,
                       int64_t n_idx, int64_t x_batch, int32_t M, int32_t N, int32_t K, int32_t n_experts,
                       int32_t transpose, int32_t group_size, int32_t bits, int32_t sorted_indices,
-                      uint16_t *y, void *workspace, size_t workspace_bytes, void *stream) {
+                      uint16_t *y, void *workspace, size_t workspace_bytes, void *stream) try {
   (void)sorted_indices;  // a hint in MLX; the segments are rebuilt here either way
   (void)x_batch;
   if (bits != 4 && bits != 8) return fail("gather_qmm: bits must be 4 or 8, got %d", bits);
@@ -575,28 +613,28 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   a.max_rows_per_expert = rows;
   MI_HIP(launch_grouped_qmm(a, false, st));
   return 0;
-}
+} MI_CATCH("gather_qmm")
 
 static size_t qmm_dense_bytes(int64_t M, int32_t K, int32_t bits, size_t *mt_words) {
   const size_t ntiles = (size_t)((M + kBigTileM - 1) / kBigTileM);
   *mt_words = tile_list_words((int)ntiles, 1);
-  size_t b = 256 + 64 + *mt_words * 4 + 256;
+  size_t b = 256 + 256 + 64 + *mt_words * 4 + 256;  // alignment of the base, the record, the tile lists
   if (bits == 4 && M >= tiled_avg_rows(bits)) b += (size_t)M * K * 2 + 256;
   return b;
 }
 
-int mi_moe_quantized_matmul_workspace_size(int64_t M, int32_t K, int32_t bits, size_t *bytes) {
+int mi_moe_quantized_matmul_workspace_size(int64_t M, int32_t K, int32_t bits, size_t *bytes) try {
   if (!bytes) return fail("quantized_matmul_workspace_size: bytes is NULL");
   if (M < 0 || K <= 0 || M * (int64_t)K > (int64_t)1 << 40) return fail("quantized_matmul_workspace_size: bad sizes");
   size_t mt = 0;
   *bytes = qmm_dense_bytes(M, K, bits, &mt);
   return 0;
-}
+} MI_CATCH("quantized_matmul_workspace_size")
 
 int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
                             const uint16_t *biases, int64_t M, int32_t N, int32_t K, int32_t transpose,
                             int32_t group_size, int32_t bits, uint16_t *y, void *workspace,
-                            size_t workspace_bytes, void *stream) {
+                            size_t workspace_bytes, void *stream) try {
   if (bits != 4 && bits != 8) return fail("quantized_matmul: bits must be 4 or 8, got %d", bits);
   if (group_size != 64) return fail("quantized_matmul: group_size must be 64, got %d", group_size);
   if (!transpose) {  // w [K, N*bits/32]: the plain kernel, no workspace
@@ -647,17 +685,17 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
   a.max_rows_per_expert = M;
   MI_HIP(launch_grouped_qmm(a, false, st));
   return 0;
-}
+} MI_CATCH("quantized_matmul")
 
-int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out, void *stream) {
+int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out, void *stream) try {
   if (n < 0) return fail("swiglu: negative element count");
   if (n == 0) return 0;
   if (!gate || !up || !out) return fail("swiglu: gate, up and out must be non-NULL");
   MI_HIP(launch_swiglu(gate, up, n, out, static_cast<hipStream_t>(stream)));
   return 0;
-}
+} MI_CATCH("swiglu")
 
-int mi_moe_stream_probe(const void *buf, size_t bytes, uint32_t *sink, void *stream) {
+int mi_moe_stream_probe(const void *buf, size_t bytes, uint32_t *sink, void *stream) try {
   if (bytes == 0) return 0;
   if (bytes % 32768) return fail("stream_probe: bytes must be a multiple of 32768, got %zu", bytes);
   if (bytes > ((size_t)1 << 34)) return fail("stream_probe: at most 16 GiB, got %zu", bytes);
@@ -665,10 +703,10 @@ int mi_moe_stream_probe(const void *buf, size_t bytes, uint32_t *sink, void *str
   if (reinterpret_cast<uintptr_t>(buf) % 16) return fail("stream_probe: buf must be 16-byte aligned");
   MI_HIP(launch_stream_probe(buf, bytes, sink, static_cast<hipStream_t>(stream)));
   return 0;
-}
+} MI_CATCH("stream_probe")
 
 int mi_moe_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *inv_perm, int64_t T,
-                   int32_t top_k, int32_t hidden, uint16_t *out, void *stream) {
+                   int32_t top_k, int32_t hidden, uint16_t *out, void *stream) try {
   if (T < 0) return fail("combine: negative token count");
   if (top_k < 1) return fail("combine: top_k must be positive, got %d", top_k);
   if (hidden <= 0 || hidden % 8) return fail("combine: hidden must be a positive multiple of 8, got %d", hidden);
@@ -677,7 +715,7 @@ int mi_moe_combine(const uint16_t *y, const uint16_t *scores, const uint32_t *in
   if (!aligned16(y) || !aligned16(out)) return fail("combine: y and out must be 16-byte aligned");
   MI_HIP(launch_combine(y, scores, inv_perm, T, top_k, hidden, nullptr, out, static_cast<hipStream_t>(stream)));
   return 0;
-}
+} MI_CATCH("combine")
 
 static int check_quant_args(const char *who, int64_t rows, int64_t cols, int32_t group_size, int32_t bits) {
   if (bits != 2 && bits != 4 && bits != 8) return fail("%s: bits must be 2, 4 or 8, got %d", who, bits);
@@ -689,21 +727,21 @@ static int check_quant_args(const char *who, int64_t rows, int64_t cols, int32_t
 }
 
 int mi_moe_quantize(const float *w, int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
-                    uint32_t *q, uint16_t *scales, uint16_t *biases, void *stream) {
+                    uint32_t *q, uint16_t *scales, uint16_t *biases, void *stream) try {
   if (check_quant_args("quantize", rows, cols, group_size, bits)) return 1;
   if (rows * cols == 0) return 0;
   if (!w || !q || !scales || !biases) return fail("quantize: w, q, scales and biases must be non-NULL");
   MI_HIP(launch_quantize(w, rows, cols, group_size, bits, q, scales, biases, static_cast<hipStream_t>(stream)));
   return 0;
-}
+} MI_CATCH("quantize")
 
 int mi_moe_dequantize(const uint32_t *q, const uint16_t *scales, const uint16_t *biases, int64_t rows,
-                      int64_t cols, int32_t group_size, int32_t bits, float *w_hat, void *stream) {
+                      int64_t cols, int32_t group_size, int32_t bits, float *w_hat, void *stream) try {
   if (check_quant_args("dequantize", rows, cols, group_size, bits)) return 1;
   if (rows * cols == 0) return 0;
   if (!q || !scales || !biases || !w_hat) return fail("dequantize: q, scales, biases and w_hat must be non-NULL");
   MI_HIP(launch_dequantize(q, scales, biases, rows, cols, group_size, bits, w_hat, static_cast<hipStream_t>(stream)));
   return 0;
-}
+} MI_CATCH("dequantize")
 
 }  // extern "C"

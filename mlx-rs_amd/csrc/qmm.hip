@@ -61,22 +61,6 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
 //
 // KW waves of a block split K chunk-wise (wave wk takes chunks wk, wk+KW, ...), the other
 // 4/KW waves take further row tiles; partial sums meet in LDS and are added in wave order.
-#ifdef MI_MOE_TRACE
-// development aid (not built by default): per-wave time stamps of the decode kernel
-__device__ unsigned long long g_trace[8 * 16384];
-#define MI_STAMP(i)                                                                          \
-  do {                                                                                       \
-    if (GLU && lane_id() == 0) {                                                             \
-      const unsigned wid = (blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6);   \
-      if (wid < 16384) g_trace[wid * 8 + (i)] = __builtin_readcyclecounter();               \
-    }                                                                                        \
-  } while (0)
-extern "C" int mi_moe_debug_read_trace(unsigned long long *host, size_t n) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), n * sizeof(unsigned long long));
-}
-#else
-#define MI_STAMP(i) do {} while (0)
-#endif
 
 #ifndef MI_MOE_RING
 #define MI_MOE_RING 4
@@ -189,7 +173,6 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   static_assert(D == MI_MOE_RING || PRECISE, "the deep ring goes with unconditional refills");
   using Regs = ChunkRegs<BITS, TWO>;
 
-  MI_STAMP(0);
   // one 64-byte record says everything about this block's segment (uniform address: scalar loads)
   const uint4 *recp = reinterpret_cast<const uint4 *>(a.work) + (size_t)blockIdx.y * 4;
   const uint4 rec0 = recp[0];
@@ -197,7 +180,6 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   const int64_t r0 = rec0.y;
   const int cnt = (int)rec0.z;
   if (cnt == 0) return;
-  MI_STAMP(6);
   const bool rec_src = a.src_in_work && rec0.w != 0u;
   constexpr int TT = BITS == 4 ? 8 : 16;        // token slots of one MFMA tile
   constexpr int TTL = TT * TG;                  // token slots of one pass
@@ -310,7 +292,6 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
           sbv[t][i] = __builtin_amdgcn_raw_buffer_load_b128((t & 1) ? br[t >> 1] : sr[t >> 1], sb_goff, i * 1024, 0);
   }
 
-  MI_STAMP(1);
   const int xstride = x_stride_bytes(sk);
   const uint32_t nib_mask = opaque_reg(0x000f000fu), nib_magic = opaque_reg(0x43004300u);  // q -> bf16 128 + q
 
@@ -549,7 +530,6 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
     };
     // the chunks [c_first, c_last) against the slab in LDS
     auto run_chunks = [&](int c_first, int c_last) __attribute__((always_inline)) {
-      MI_STAMP(4);
       // D chunks in flight: slot d is refilled as soon as its chunk has been consumed.
       if constexpr (PRECISE) {
         int base = c_first;
@@ -588,9 +568,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
       if (!PRE || t0 > 0) __syncthreads();  // zero fill done / every wave is done reading the previous tile
       if (t0 > 0) reprime();
       stage_rows(0, K);
-      MI_STAMP(2);
       __syncthreads();
-      MI_STAMP(3);
       after_stage(0);
       run_chunks(ch0, ch1);
     } else {
@@ -610,7 +588,6 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
       }
     }
 
-    MI_STAMP(5);
     if constexpr (BITS == 4) {  // rows 8-15 (second group of each chunk) onto rows 0-7
 #pragma unroll
       for (int g = 0; g < TG; ++g)

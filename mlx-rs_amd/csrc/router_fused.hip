@@ -11,6 +11,21 @@
 // with device-coherent stores and read with device-coherent loads; a workgroup waits for its own
 // stores to be acknowledged before it counts itself in.  No cache-wide write-back or invalidate
 // is involved (on this chip those cost microseconds per workgroup).
+//
+// Why this is safe on gfx950 although it is below what the HIP memory model promises:
+//  * an `sc1` store is written through the issuing XCD's L2 to memory, and its acknowledgement
+//    (what `s_waitcnt vmcnt(0)` waits for) comes back only when the data is there; an `sc1`
+//    load is served from memory, not from a line another XCD's L2 may hold stale.  So a value whose
+//    store was acknowledged is what any later `sc1` load on any XCD returns;
+//  * the counters are device-scope atomics, executed at the memory side: every workgroup sees one
+//    order of them;
+//  * therefore: wave stores (sc1) -> every wave waits vmcnt(0) -> barrier -> one thread's atomic
+//    increment.  The workgroup that observes the full count runs after every contributor's
+//    increment, hence after every contributor's acknowledged stores, and reads them with sc1 loads
+//    issued after its own barrier (no earlier load of those addresses exists in the workgroup, so
+//    nothing stale sits in its registers, and sc1 loads do not hit in the per-CU cache).
+// The wait is written out (`wait_own_stores`): a workgroup-scope release fence does not make the
+// compiler emit it when the workgroup runs on one CU.
 // The counters return to zero before the kernel ends, so the next launch finds them ready.
 // Results are those of the separate kernels bit for bit (same device functions, and none of
 // them depends on which workgroup runs it).
@@ -18,6 +33,9 @@
 #include "router_dev.hpp"
 
 namespace mi_moe {
+
+// every vector-memory operation of this wave, stores included, has been acknowledged
+__device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // counters[0]: tokens selected; counters[1 + t]: logit workgroups of token t that have finished
 template <int NV>
@@ -45,7 +63,8 @@ __global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
       store_agent(logits + (int64_t)t * E + e, f32_to_bf16((float)s));
     }
   }
-  // every wave's store has been acknowledged (workgroup-scope release = wait for own stores) ...
+  // every wave's stores (the logit, the normalised row) have been acknowledged ...
+  wait_own_stores();
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (tid == 0) {  // ... before the workgroup is counted in
@@ -60,6 +79,7 @@ __global__ __launch_bounds__(kDispThreads) void router_fused_kernel(
   if (wave == 0)
     select_wave<NV, true>(logits + (int64_t)t * E, E, k, mode, topk_idx + (int64_t)t * k,
                           topk_w + (int64_t)t * k);
+  wait_own_stores();  // the selected experts are where the dispatching workgroup will read them
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (tid == 0) {

@@ -196,52 +196,185 @@ pub mod fast {
 
 pub mod nn {
     use super::*;
+    use mlx_rs::macros::{ModuleParameters, Quantizable};
+    use mlx_rs::module::ModuleParameters as _; // freeze_parameters
+    use mlx_rs::nn::Linear;
+    use mlx_rs::quantization::{MaybeQuantized, Quantizable};
     use std::marker::PhantomData;
 
-    /// One bank of E quantized matrices: the fields of `QuantizedLinear`
-    /// (`mlx-rs/src/nn/quantized.rs:254-279`) with a leading expert axis, named as
-    /// `mlx_lm.convert` writes them (`…switch_mlp.gate_proj.{weight,scales,biases}`).
-    #[derive(Debug, Clone)]
+    /// One bank of E dense matrices `[E, N, K]`: what a switch layer holds before quantisation
+    /// (the role `Linear` has for `QuantizedLinear`, `mlx-rs/src/nn/linear.rs:60-110`).
+    /// This library has no dense expert product; the type exists so that the block can be built
+    /// dense and quantised in process (`nn::quantize(model, None, None)`,
+    /// `mlx-rs/src/nn/quantized.rs:25-36`, `examples/mistral/src/main.rs:186-193`).
+    #[derive(Debug, Clone, ModuleParameters)]
+    pub struct SwitchLinear {
+        #[param]
+        pub weight: Param<Array>, // [E, N, K]
+    }
+
+    /// One bank of E quantized matrices: the parameters of `QuantizedLinear`
+    /// (`mlx-rs/src/nn/quantized.rs:254-279`) with a leading expert axis.  The packed weight is a
+    /// parameter of this struct itself, so the flattened keys are the ones `mlx_lm.convert`
+    /// writes (`...switch_mlp.gate_proj.{weight,scales,biases}`); `QuantizedLinear` nests it as
+    /// `inner.weight` (`nn/quantized.rs:325-327`).
+    #[derive(Debug, Clone, ModuleParameters)]
     pub struct QuantizedSwitchLinear {
+        pub group_size: i32,
+        pub bits: i32,
+
+        #[param]
         pub weight: Param<Array>, // u32 [E, N, K*bits/32]
+
+        #[param]
         pub scales: Param<Array>, // bf16 [E, N, K/group_size]
+
+        #[param]
         pub biases: Param<Array>, // bf16 [E, N, K/group_size]
     }
 
-    #[derive(Debug, Clone)]
-    pub struct SwitchGlu {
-        pub gate_proj: QuantizedSwitchLinear,
-        pub up_proj: QuantizedSwitchLinear,
-        pub down_proj: QuantizedSwitchLinear,
+    impl QuantizedSwitchLinear {
+        /// Containers of the right shapes for a checkpoint to be loaded into
+        /// (`load_safetensors` only overwrites parameters that exist, `module/module.rs:260-283`).
+        pub fn zeros(n_experts: i32, n: i32, k: i32, group_size: i32, bits: i32) -> Result<Self, Exception> {
+            let mut q = Self {
+                group_size,
+                bits,
+                weight: Param::new(Array::zeros::<u32>(&[n_experts, n, k * bits / 32])?),
+                scales: Param::new(Array::zeros::<half::bf16>(&[n_experts, n, k / group_size])?),
+                biases: Param::new(Array::zeros::<half::bf16>(&[n_experts, n, k / group_size])?),
+            };
+            q.freeze_parameters(true); // as QuantizedLinear, nn/quantized.rs:275-276
+            Ok(q)
+        }
     }
 
-    /// Router + experts; `forward` is one library call.  In `mlx-lm` this struct additionally
-    /// derives `ModuleParameters` with `#[param]` on `gate` and `switch_mlp` so that
-    /// `load_safetensors` (`mlx-rs/src/module/module.rs:260-283`) finds
-    /// `mlp.gate.weight` and `mlp.switch_mlp.*`.
+    impl Quantizable for SwitchLinear {
+        type Quantized = QuantizedSwitchLinear;
+        type QuantizationError = Exception;
+
+        /// Every row of every expert is quantised on its own, so the bank goes through
+        /// `ops::quantize` (`mlx-rs/src/ops/quantization.rs:50-83`) as it is.
+        fn try_into_quantized(self, group_size: i32, bits: i32) -> Result<QuantizedSwitchLinear, Exception> {
+            let w = self.weight.value.as_dtype(Dtype::Bfloat16)?;
+            let (wq, scales, biases) = mlx_rs::ops::quantize(&w, group_size, bits)?;
+            let mut q = QuantizedSwitchLinear { group_size, bits, weight: Param::new(wq), scales: Param::new(scales), biases: Param::new(biases) };
+            q.freeze_parameters(true);
+            Ok(q)
+        }
+    }
+
+    /// The three expert banks of a SwiGLU switch layer, with mlx-lm's field names.
+    #[derive(Debug, Clone, ModuleParameters, Quantizable)]
+    pub struct SwitchGlu {
+        #[quantizable]
+        #[param]
+        pub gate_proj: MaybeQuantized<SwitchLinear>,
+
+        #[quantizable]
+        #[param]
+        pub up_proj: MaybeQuantized<SwitchLinear>,
+
+        #[quantizable]
+        #[param]
+        pub down_proj: MaybeQuantized<SwitchLinear>,
+    }
+
+    /// The library handle and what it was created from.  Kept apart from the block so that the
+    /// block itself has no `Drop` (the derived `Quantizable` moves the fields out of `self`,
+    /// `mlx-macros/src/quantizable.rs:76-88`).
     #[derive(Debug)]
+    struct Bound {
+        handle: sys::mi_moe_handle,
+        pointers: [usize; 11], // device addresses of the ten weight arrays and the router bias
+        config: [i32; 7],
+    }
+
+    impl Drop for Bound {
+        fn drop(&mut self) {
+            if !self.handle.is_null() {
+                unsafe { sys::mi_moe_destroy(self.handle) };
+            }
+        }
+    }
+
+    /// Router + experts where the dense `Mlp` stands in a decoder layer
+    /// (`mlx-lm/src/models/qwen3.rs:204-255`, field `mlp` of `TransformerBlock`, `:257-275`):
+    /// the flattened parameter keys below `mlp.` are `gate.weight` (and `gate.bias` when the
+    /// router has one) and `switch_mlp.{gate_proj,up_proj,down_proj}.{weight,scales,biases}`.
+    /// `forward` is one library call.
+    #[derive(Debug, ModuleParameters, Quantizable)]
     pub struct SparseMoeBlock<D: DeviceAccess> {
-        pub gate: Param<Array>, // bf16 [E, H], bias-free Linear (mlx-rs/src/nn/linear.rs:84-96)
+        /// bias-free `Linear` `[E, H]` in bf16, never quantised (`mlx-rs/src/nn/linear.rs:84-96`);
+        /// a bias, if present, is added to the logits before they are rounded to bf16
+        #[param]
+        pub gate: Linear,
+
+        #[quantizable]
+        #[param]
         pub switch_mlp: SwitchGlu,
+
         pub top_k: i32,
         pub norm_topk_prob: bool,
         pub softmax_after_topk: bool, // Mixtral
-        pub bits: i32,
-        pub group_size: i32,
-        handle: sys::mi_moe_handle,
+        pub stream: Stream,
+
+        bound: Option<Bound>,
+        router_bias_f32: Option<Array>, // gate.bias as float32, the form the library takes
         workspace: Option<Array>,
         workspace_tokens: i64,
-        stream: Stream,
         _d: PhantomData<D>,
     }
 
     impl<D: DeviceAccess> SparseMoeBlock<D> {
-        #[allow(clippy::too_many_arguments)]
-        pub fn new(gate: Array, switch_mlp: SwitchGlu, top_k: i32, norm_topk_prob: bool, softmax_after_topk: bool, bits: i32, group_size: i32, stream: Stream) -> Self {
-            Self { gate: Param::new(gate), switch_mlp, top_k, norm_topk_prob, softmax_after_topk, bits, group_size, handle: std::ptr::null_mut(), workspace: None, workspace_tokens: 0, stream, _d: PhantomData }
+        pub fn new(gate: Linear, switch_mlp: SwitchGlu, top_k: i32, norm_topk_prob: bool, softmax_after_topk: bool, stream: Stream) -> Self {
+            Self { gate, switch_mlp, top_k, norm_topk_prob, softmax_after_topk, stream, bound: None, router_bias_f32: None, workspace: None, workspace_tokens: 0, _d: PhantomData }
         }
 
-        fn config(&self) -> sys::mi_moe_config {
+        /// A block with zero-filled quantized containers, ready for
+        /// `load_safetensors` of a quantized checkpoint (`module/module.rs:260-283`).
+        #[allow(clippy::too_many_arguments)]
+        pub fn new_quantized(hidden: i32, n_experts: i32, intermediate: i32, top_k: i32, norm_topk_prob: bool, softmax_after_topk: bool, group_size: i32, bits: i32, stream: Stream) -> Result<Self, Exception> {
+            let gate = Linear { weight: Param::new(Array::zeros::<half::bf16>(&[n_experts, hidden])?), bias: Param::new(None) };
+            let bank = |n, k| QuantizedSwitchLinear::zeros(n_experts, n, k, group_size, bits).map(MaybeQuantized::Quantized);
+            let switch_mlp = SwitchGlu { gate_proj: bank(intermediate, hidden)?, up_proj: bank(intermediate, hidden)?, down_proj: bank(hidden, intermediate)? };
+            Ok(Self::new(gate, switch_mlp, top_k, norm_topk_prob, softmax_after_topk, stream))
+        }
+
+        fn quantized(m: &MaybeQuantized<SwitchLinear>, what: &str) -> Result<&QuantizedSwitchLinear, Exception> {
+            match m {
+                MaybeQuantized::Quantized(q) => Ok(q),
+                MaybeQuantized::Original(_) => Err(Exception::custom(format!(
+                    "[mi_moe] {what} is not quantized: this path runs MLX-affine 4/8-bit experts only; \
+                     quantize the block (nn::quantize) or load a quantized checkpoint"
+                ))),
+            }
+        }
+
+        fn qmat(m: &QuantizedSwitchLinear) -> Result<sys::mi_moe_qmat, Exception> {
+            expect_dtype(&m.weight, Dtype::Uint32, "weight")?;
+            expect_dtype(&m.scales, Dtype::Bfloat16, "scales")?;
+            expect_dtype(&m.biases, Dtype::Bfloat16, "biases")?;
+            m.weight.eval()?;
+            m.scales.eval()?;
+            m.biases.eval()?;
+            Ok(sys::mi_moe_qmat { w: D::device_ptr(&m.weight) as *const u32, scales: D::device_ptr(&m.scales) as *const u16, biases: D::device_ptr(&m.biases) as *const u16 })
+        }
+
+        /// Binds the weights and sizes the workspace for `t` tokens.  The handle keeps device
+        /// addresses, so it is created again whenever a parameter has been replaced since
+        /// (`load_safetensors`, `update`: `module/module.rs:70-80,260-283` assign new arrays).
+        fn ensure(&mut self, t: i64) -> Result<(), Exception> {
+            let (g, u, d) = (
+                Self::quantized(&self.switch_mlp.gate_proj, "switch_mlp.gate_proj")?,
+                Self::quantized(&self.switch_mlp.up_proj, "switch_mlp.up_proj")?,
+                Self::quantized(&self.switch_mlp.down_proj, "switch_mlp.down_proj")?,
+            );
+            if g.bits != u.bits || g.bits != d.bits || g.group_size != u.group_size || g.group_size != d.group_size {
+                return Err(Exception::custom("[mi_moe] the three expert banks must share bits and group_size"));
+            }
+            expect_dtype(&self.gate.weight, Dtype::Bfloat16, "gate.weight")?;
+            self.gate.weight.eval()?;
             let score_mode = if self.softmax_after_topk {
                 sys::MI_MOE_SCORE_TOPK_THEN_SOFTMAX
             } else if self.norm_topk_prob {
@@ -249,39 +382,53 @@ pub mod nn {
             } else {
                 sys::MI_MOE_SCORE_SOFTMAX_THEN_TOPK
             };
-            sys::mi_moe_config {
-                hidden: self.gate.dim(1),
-                n_experts: self.gate.dim(0),
+            let cfg = sys::mi_moe_config {
+                hidden: self.gate.weight.dim(1),
+                n_experts: self.gate.weight.dim(0),
                 top_k: self.top_k,
-                intermediate: self.switch_mlp.gate_proj.weight.dim(1),
-                bits: self.bits,
-                group_size: self.group_size,
+                intermediate: g.weight.dim(1),
+                bits: g.bits,
+                group_size: g.group_size,
                 score_mode,
-            }
-        }
-
-        fn qmat(m: &QuantizedSwitchLinear) -> Result<sys::mi_moe_qmat, Exception> {
-            m.weight.eval()?;
-            m.scales.eval()?;
-            m.biases.eval()?;
-            Ok(sys::mi_moe_qmat { w: D::device_ptr(&m.weight) as *const u32, scales: D::device_ptr(&m.scales) as *const u16, biases: D::device_ptr(&m.biases) as *const u16 })
-        }
-
-        /// Binds the weights (once) and sizes the workspace for `t` tokens (when `t` grows).
-        fn ensure(&mut self, t: i64) -> Result<(), Exception> {
-            let cfg = self.config();
-            if self.handle.is_null() {
-                self.gate.eval()?;
-                let w = sys::mi_moe_weights {
-                    router_w: D::device_ptr(&self.gate) as *const u16,
-                    router_bias: std::ptr::null(),
-                    gate: Self::qmat(&self.switch_mlp.gate_proj)?,
-                    up: Self::qmat(&self.switch_mlp.up_proj)?,
-                    down: Self::qmat(&self.switch_mlp.down_proj)?,
+            };
+            // the router's bias, once per distinct bias array, as float32
+            let bias_src = self.gate.bias.value.as_ref().map(|b| D::device_ptr(b) as usize).unwrap_or(0);
+            let bias_bound = self.bound.as_ref().map(|b| b.pointers[10]).unwrap_or(usize::MAX);
+            if bias_src != bias_bound {
+                self.router_bias_f32 = match self.gate.bias.value.as_ref() {
+                    Some(b) => {
+                        let f = b.as_dtype(Dtype::Float32)?;
+                        f.eval()?;
+                        Some(f)
+                    }
+                    None => None,
                 };
-                check(unsafe { sys::mi_moe_create(&cfg, &w, &mut self.handle) })?;
             }
-            if t > self.workspace_tokens {
+            let w = sys::mi_moe_weights {
+                router_w: D::device_ptr(&self.gate.weight) as *const u16,
+                router_bias: self.router_bias_f32.as_ref().map(|b| D::device_ptr(b) as *const f32).unwrap_or(std::ptr::null()),
+                gate: Self::qmat(g)?,
+                up: Self::qmat(u)?,
+                down: Self::qmat(d)?,
+            };
+            let pointers = [
+                w.router_w as usize, w.gate.w as usize, w.gate.scales as usize, w.gate.biases as usize,
+                w.up.w as usize, w.up.scales as usize, w.up.biases as usize,
+                w.down.w as usize, w.down.scales as usize, w.down.biases as usize, bias_src,
+            ];
+            let config = [cfg.hidden, cfg.n_experts, cfg.top_k, cfg.intermediate, cfg.bits, cfg.group_size, cfg.score_mode];
+            let stale = match &self.bound {
+                Some(b) => b.pointers != pointers || b.config != config,
+                None => true,
+            };
+            if stale {
+                self.bound = None; // destroys the old handle
+                let mut handle: sys::mi_moe_handle = std::ptr::null_mut();
+                check(unsafe { sys::mi_moe_create(&cfg, &w, &mut handle) })?;
+                self.bound = Some(Bound { handle, pointers, config });
+                self.workspace_tokens = 0; // the size depends on the configuration
+            }
+            if t > self.workspace_tokens || self.workspace.is_none() {
                 let mut bytes = 0usize;
                 check(unsafe { sys::mi_moe_workspace_size(&cfg, t, &mut bytes) })?;
                 self.workspace = Some(D::device_buffer(bytes)?);
@@ -298,16 +445,18 @@ pub mod nn {
         /// (`mlx-lm/src/models/qwen3.rs:310-325`).
         pub fn forward_residual(&mut self, h: &Array, norm_weight: &Array, eps: f32) -> Result<Array, Exception> {
             expect_dtype(h, Dtype::Bfloat16, "h")?;
+            expect_dtype(norm_weight, Dtype::Bfloat16, "norm_weight")?;
             h.eval()?;
             norm_weight.eval()?;
             let t = Self::tokens(h);
             self.ensure(t)?;
             let mut out = Array::zeros::<half::bf16>(h.shape())?;
             out.eval()?;
+            let handle = self.bound.as_ref().unwrap().handle;
             let ws = self.workspace.as_mut().unwrap();
             let ws_bytes = ws.nbytes();
             check(unsafe {
-                sys::mi_moe_forward_residual(self.handle, D::device_ptr(h) as *const u16, D::device_ptr(norm_weight) as *const u16, eps, t, D::device_ptr_mut(&mut out) as *mut u16, D::device_ptr_mut(ws), ws_bytes, std::ptr::null(), D::hip_stream(&self.stream))
+                sys::mi_moe_forward_residual(handle, D::device_ptr(h) as *const u16, D::device_ptr(norm_weight) as *const u16, eps, t, D::device_ptr_mut(&mut out) as *mut u16, D::device_ptr_mut(ws), ws_bytes, std::ptr::null(), D::hip_stream(&self.stream))
             })?;
             Ok(out)
         }
@@ -325,22 +474,19 @@ pub mod nn {
             self.ensure(t)?;
             let mut out = Array::zeros::<half::bf16>(x.shape())?;
             out.eval()?;
+            let handle = self.bound.as_ref().unwrap().handle;
             let ws = self.workspace.as_mut().unwrap();
             let ws_bytes = ws.nbytes();
             check(unsafe {
-                sys::mi_moe_forward(self.handle, D::device_ptr(x) as *const u16, t, D::device_ptr_mut(&mut out) as *mut u16, D::device_ptr_mut(ws), ws_bytes, std::ptr::null(), D::hip_stream(&self.stream))
+                sys::mi_moe_forward(handle, D::device_ptr(x) as *const u16, t, D::device_ptr_mut(&mut out) as *mut u16, D::device_ptr_mut(ws), ws_bytes, std::ptr::null(), D::hip_stream(&self.stream))
             })?;
             Ok(out)
         }
 
-        fn training_mode(&mut self, _mode: bool) {} // frozen weights, as QuantizedLinear (nn/quantized.rs:275-276)
-    }
-
-    impl<D: DeviceAccess> Drop for SparseMoeBlock<D> {
-        fn drop(&mut self) {
-            if !self.handle.is_null() {
-                unsafe { sys::mi_moe_destroy(self.handle) };
-            }
+        /// Nothing in the block depends on the mode; the router is told, as `Mlp` tells its
+        /// layers (`mlx-lm/src/models/qwen3.rs:249-254`).
+        fn training_mode(&mut self, mode: bool) {
+            self.gate.training_mode(mode);
         }
     }
 }

@@ -29,7 +29,6 @@ def _run_case(orc, H, E, k, I, bits, T, score_mode, seed=0, zipf_s=None, threads
     got = bits_u16(out)
     mf, rf = assert_close_bf16(got, ref_f, what="vs oracle (fused rounding points)")
     ms, rs = assert_close_bf16(got, ref_s, what="vs oracle (op-by-op rounding)")
-    print(f"  fused: max-abs {mf:.2e} rel-fro {rf:.2e}; strict: max-abs {ms:.2e} rel-fro {rs:.2e}", flush=True)
     return got
 
 
@@ -120,9 +119,8 @@ def test_tile_classes(orc, T, E, k, bits, zipf):
 def test_tile_classes_with_the_chip_full(orc, bits, zipf):
     # narrow layers leave the chip blocks to spare and run their 256- and 128-row tiles with the
     # 64-row kernel (the shapes of test_tile_classes); here both products have more than 256 blocks
-    # even with 128-row tiles, so each list is run by the kernel of its own size (weights of half the
-    # usual spread: the absolute bar is meant for outputs of magnitude 1, these rows are 3072 long)
-    _run_case(orc, 3072, 8, 2, 1536, bits, 1100, 0, seed=17 + bits, zipf_s=zipf, std=0.01)
+    # even with 128-row tiles, so each list is run by the kernel of its own size
+    _run_case(orc, 3072, 8, 2, 1536, bits, 1100, 0, seed=17 + bits, zipf_s=zipf)
 
 
 @pytest.mark.parametrize("T,H,I", [(40, 2048, 768), (44, 1024, 2048), (13, 256, 384), (16, 2048, 256)])
@@ -162,14 +160,13 @@ def test_norm_and_residual_around_the_block(orc, T, H, E, k, I, bits, mode, zipf
     for name in ("topk_idx", "counts", "perm"):
         assert np.array_equal(bits_u32(dbg[name]).reshape(d[name].shape), d[name]), name
     assert np.array_equal(bits_u16(dbg["topk_w"]), d["topk_w"])
-    scale = max(1.0, float(np.abs(f32_of_bits(ref_s)).max()) / 4)  # |x| reaches 4: one bf16 ulp there is 3e-2
-    assert_close_bf16(bits_u16(out), ref_f, max_abs=2e-2 * scale, what="vs oracle (fused rounding points)")
-    assert_close_bf16(bits_u16(out), ref_s, max_abs=2e-2 * scale, what="vs oracle (op-by-op rounding)")
+    assert_close_bf16(bits_u16(out), ref_f, what="vs oracle (fused rounding points)")
+    assert_close_bf16(bits_u16(out), ref_s, what="vs oracle (op-by-op rounding)")
     # and it is the plain forward on rms_norm(x) plus x, up to the one rounding that is saved
     y = blk.forward(xn)
     torch.cuda.synchronize()
     want = (xd.float() + y.float()).bfloat16()
-    assert (out.float() - want.float()).abs().max().item() <= 2e-2 * scale
+    assert_close_bf16(bits_u16(out), bits_u16(want), what="vs x + forward(rms_norm(x)) in two roundings")
     with pytest.raises(m.MoeError, match="alias"):
         blk.forward_residual(xd, nwd, 1e-6, out=xd)
 
@@ -253,3 +250,10 @@ def test_empty_batch_and_leading_axes(orc):
     assert empty.shape == (0, H)
     out, dbg = blk.forward(x[:0].reshape(0, 1, H), debug=True)
     assert out.shape == (0, 1, H) and dbg["perm"].numel() == 0
+
+
+@pytest.mark.parametrize("T,zipf", [(16, None), (60, 1.3), (200, 1.3)])
+def test_widest_outputs_of_the_shape_sweep(orc, T, zipf):
+    # the shape whose outputs are the largest of those swept (rows of 4096 values, two experts per
+    # token: |out| reaches 2.7, where a bf16 ulp is 1.6e-2), under the one tolerance rule
+    _run_case(orc, 4096, 8, 2, 1024, 4, T, 0, seed=200 + T, zipf_s=zipf)

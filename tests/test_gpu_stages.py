@@ -118,7 +118,7 @@ def test_swiglu_and_combine(orc, m):
     u = orc.f32_to_bf16(np.clip(rng.normal(0, 0.9, (77, 96)), -1.9, 1.9).astype(np.float32))
     got = m.ops.swiglu(bf16_tensor(g, "cuda"), bf16_tensor(u, "cuda"))
     assert_close_bf16(bits_u16(got), orc.swiglu_bf16(g, u), what="swiglu vs op-by-op oracle")
-    assert_close_bf16(bits_u16(got), orc.swiglu_f32(f32_of_bits(g), f32_of_bits(u)), max_abs=2e-2, rel_fro=3e-3,
+    assert_close_bf16(bits_u16(got), orc.swiglu_f32(f32_of_bits(g), f32_of_bits(u)), rel_fro=3e-3,
                       what="swiglu vs single-rounding oracle")
     T, k, H = 50, 8, 2048
     y = orc.f32_to_bf16(rng.normal(0, 1, (T * k, H)).astype(np.float32))

@@ -124,3 +124,70 @@ def test_library_exports_what_the_binding_links():
     rf, _, _ = parse_rust()
     for name in rf:
         assert hasattr(lib, name), name
+
+
+# ---------------------------------------------------------------- the safe layer (mi-moe)
+SAFE = os.path.join(ROOT, "mlx-rs_amd", "rust", "mi-moe", "src", "lib.rs")
+
+
+def _safe_source():
+    return re.sub(r"//.*", "", open(SAFE).read())
+
+
+def _structs_with_derives(src):
+    """{struct name: (set of derived traits, body text)}"""
+    out = {}
+    for m in re.finditer(r"((?:#\[[^\]]*\]\s*)*)(?:pub\s+)?struct\s+(\w+)\s*(?:<[^>{]*>)?\s*\{(.*?)\n    \}", src, flags=re.S):
+        derives = set()
+        for d in re.finditer(r"#\[derive\(([^)]*)\)\]", m.group(1)):
+            derives.update(t.strip() for t in d.group(1).split(","))
+        out[m.group(2)] = (derives, m.group(3))
+    return out
+
+
+def test_every_module_also_has_module_parameters():
+    """`trait Module<Input>: ModuleParameters + Debug` (mlx-rs/src/module/module.rs:28): a type given
+    an `impl Module` must derive (or implement) ModuleParameters and Debug, or it cannot compile."""
+    src = _safe_source()
+    structs = _structs_with_derives(src)
+    impls = re.findall(r"impl\s*(?:<[^>]*>)?\s*Module<[^>]*>\s+for\s+(\w+)", src)
+    assert impls, "no impl Module found"
+    for name in impls:
+        derives, _ = structs[name]
+        has_mp = "ModuleParameters" in derives or re.search(r"impl[^{]*\bModuleParameters\s+for\s+%s\b" % name, src)
+        assert has_mp, f"{name} implements Module but not ModuleParameters"
+        assert "Debug" in derives, f"{name} implements Module but not Debug"
+
+
+def test_parameter_fields_follow_the_checkpoint_names():
+    """The flattened keys are the field names joined by dots (mlx-macros/src/module_parameters.rs:97-101):
+    gate.weight and switch_mlp.{gate_proj,up_proj,down_proj}.{weight,scales,biases}."""
+    structs = _structs_with_derives(_safe_source())
+
+    def params(name):
+        return re.findall(r"#\[param\]\s*pub\s+(\w+)\s*:", structs[name][1])
+
+    assert params("SparseMoeBlock") == ["gate", "switch_mlp"]
+    assert params("SwitchGlu") == ["gate_proj", "up_proj", "down_proj"]
+    assert params("QuantizedSwitchLinear") == ["weight", "scales", "biases"]
+    assert params("SwitchLinear") == ["weight"]
+    for name in ("SparseMoeBlock", "SwitchGlu", "QuantizedSwitchLinear", "SwitchLinear"):
+        assert "ModuleParameters" in structs[name][0], name
+
+
+def test_derived_quantizable_types_can_be_taken_apart():
+    """derive(Quantizable) rebuilds the struct from its moved-out fields
+    (mlx-macros/src/quantizable.rs:76-88): such a type needs a #[quantizable] field and no Drop."""
+    src = _safe_source()
+    structs = _structs_with_derives(src)
+    derived = [n for n, (d, _) in structs.items() if "Quantizable" in d]
+    assert sorted(derived) == ["SparseMoeBlock", "SwitchGlu"]
+    for name in derived:
+        assert "#[quantizable]" in structs[name][1], f"{name} has no quantizable field"
+        assert not re.search(r"impl\s*(?:<[^>]*>)?\s*Drop\s+for\s+%s\b" % name, src), f"{name} implements Drop"
+
+
+def test_the_router_bias_reaches_the_library():
+    src = _safe_source()
+    assert "router_bias: std::ptr::null()" not in src
+    assert re.search(r"router_bias:\s*self\.router_bias_f32", src)

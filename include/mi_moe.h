@@ -129,11 +129,18 @@ int mi_moe_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_
 /* The same forward with a HIP event recorded on `stream` before the first launch and
  * after each stage; waits for the last one and returns the MI_MOE_N_STAGES elapsed times
  * in milliseconds (host array): router logits, router select, dispatch, gate/up + SwiGLU,
- * down, combine.  For measurement; mlx-rs has no counterpart (it times with
+ * down, combine (an event pair adds several microseconds to what lies between).  kernel_ms (host
+ * array of MI_MOE_N_KERNEL_TIMES, or NULL): the durations of the grouped-product kernels themselves,
+ * each from the start and end time stamps of its own dispatch (what a profiler reports for the
+ * kernel): gate/up + SwiGLU over the 256-row, 128-row and 64-row tile lists and over the streamed
+ * segments, then the down product over the same four; 0 where no kernel was launched.  The kernels
+ * run one after the other on `stream`.  For measurement; mlx-rs has no counterpart (it times with
  * Instant::now() around eval, mlx-rs/examples/linear_regression.rs:40-59). */
 #define MI_MOE_N_STAGES 6
+#define MI_MOE_N_KERNEL_TIMES 8
 int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
-                         void *workspace, size_t workspace_bytes, void *stream, float *stage_ms);
+                         void *workspace, size_t workspace_bytes, void *stream, float *stage_ms,
+                         float *kernel_ms);
 
 /* ---- R1-R4 router: gate Linear + softmax(precise) + argpartition top-k +
  * take_along_axis + renormalise (mlx_matmul, mlx_softmax_axis, mlx_argpartition_axis,

@@ -9,6 +9,9 @@ SCORE_SOFTMAX_THEN_TOPK_RENORM = 0
 SCORE_SOFTMAX_THEN_TOPK = 1
 SCORE_TOPK_THEN_SOFTMAX = 2
 N_STAGES = 6
+N_KERNEL_TIMES = 8
+KERNEL_NAMES = ("gate_up_tiles256", "gate_up_tiles128", "gate_up_tiles64", "gate_up_streamed",
+                "down_tiles256", "down_tiles128", "down_tiles64", "down_streamed")
 STAGE_NAMES = ("router_logits", "router_select", "dispatch", "gate_up_swiglu", "down", "combine")
 
 # every symbol include/mi_moe.h declares
@@ -84,7 +87,7 @@ def load_library():
         "mi_moe_destroy": [vp],
         "mi_moe_workspace_size": [C.POINTER(Config), i64, C.POINTER(sz)],
         "mi_moe_forward": [vp, vp, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
-        "mi_moe_forward_timed": [vp, vp, i64, vp, vp, sz, vp, C.POINTER(C.c_float)],
+        "mi_moe_forward_timed": [vp, vp, i64, vp, vp, sz, vp, C.POINTER(C.c_float), C.POINTER(C.c_float)],
         "mi_moe_forward_residual": [vp, vp, vp, C.c_float, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
         "mi_moe_rms_norm": [vp, vp, C.c_float, i64, i32, vp, vp],
         "mi_moe_route_workspace_size": [i32, i64, C.POINTER(sz)],

@@ -244,9 +244,11 @@ int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *
 
 // The launch sequence of one forward.  ev: nullptr, or kStages + 1 events recorded on the
 // stream before the first launch and after each stage.
+// kt: nullptr, or MI_MOE_N_KERNEL_TIMES timers for the grouped-product kernels (with ev).
 static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16_t *out, void *workspace,
                         size_t workspace_bytes, const mi_moe_debug_out *dbg, hipStream_t st,
-                        hipEvent_t *ev, const uint16_t *norm_weight = nullptr, float eps = 0.f) {
+                        hipEvent_t *ev, const uint16_t *norm_weight = nullptr, float eps = 0.f,
+                        KernelTimer *kt = nullptr) {
   const uint16_t *x = x_in;
   if (!h) return fail("forward: handle is NULL");
   if (T < 0) return fail("forward: negative token count");
@@ -407,6 +409,25 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     }
     if (rc) return rc;
     MI_HIP(je);
+  } else if (kt) {
+    // one kernel after the other, each dispatch with a timer of its own: tile classes 0, 1, 2 (the
+    // 256-, 128- and 64-row lists), then the streamed segments; gate/up first, then down
+    struct TimerScope {  // the timer never outlives the launch it is meant for
+      explicit TimerScope(KernelTimer *t) { g_kernel_timer = t; }
+      ~TimerScope() { g_kernel_timer = nullptr; }
+    };
+    for (int half = 0; half < 2; ++half) {
+      const GroupedArgs &g = half == 0 ? a : d;
+      for (int cls = 0; cls < 3; ++cls) {
+        TimerScope scope(&kt[4 * half + cls]);
+        MI_HIP(launch_large_qmm_class(g, half == 0, cls, st));
+      }
+      {
+        TimerScope scope(&kt[4 * half + 3]);
+        MI_HIP(launch_small_qmm(g, half == 0, st));
+      }
+      MI_STAGE_DONE();
+    }
   } else {
     MI_HIP(launch_grouped_qmm(a, true, st));
     MI_STAGE_DONE();
@@ -456,18 +477,26 @@ int mi_moe_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_
 } MI_CATCH("rms_norm")
 
 int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
-                         size_t workspace_bytes, void *stream, float *stage_ms) try {
+                         size_t workspace_bytes, void *stream, float *stage_ms, float *kernel_ms) try {
   if (!stage_ms) return fail("forward_timed: stage_ms is NULL");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipEvent_t ev[MI_MOE_N_STAGES + 1];
-  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) {
+  constexpr int kEvents = MI_MOE_N_STAGES + 1 + 2 * MI_MOE_N_KERNEL_TIMES;
+  hipEvent_t ev[kEvents];
+  for (int i = 0; i < kEvents; ++i) {
     const hipError_t e = hipEventCreate(&ev[i]);
     if (e != hipSuccess) {
       while (--i >= 0) (void)hipEventDestroy(ev[i]);
       return hip_fail("hipEventCreate", e);
     }
   }
-  int rc = forward_impl(h, x, T, out, workspace, workspace_bytes, nullptr, st, ev);
+  KernelTimer kt[MI_MOE_N_KERNEL_TIMES];
+  for (int i = 0; i < MI_MOE_N_KERNEL_TIMES; ++i) {
+    kt[i].start = ev[MI_MOE_N_STAGES + 1 + 2 * i];
+    kt[i].stop = ev[MI_MOE_N_STAGES + 2 + 2 * i];
+  }
+  int rc = forward_impl(h, x, T, out, workspace, workspace_bytes, nullptr, st, ev, nullptr, 0.f, kt);
+  if (kernel_ms)
+    for (int i = 0; i < MI_MOE_N_KERNEL_TIMES; ++i) kernel_ms[i] = 0.f;
   if (rc == 0 && T > 0) {
     hipError_t e = hipEventSynchronize(ev[MI_MOE_N_STAGES]);
     if (e != hipSuccess) rc = hip_fail("hipEventSynchronize", e);
@@ -475,8 +504,13 @@ int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t
       e = hipEventElapsedTime(&stage_ms[i], ev[i], ev[i + 1]);
       if (e != hipSuccess) rc = hip_fail("hipEventElapsedTime", e);
     }
+    for (int i = 0; rc == 0 && kernel_ms && i < MI_MOE_N_KERNEL_TIMES; ++i) {
+      if (!kt[i].used) continue;
+      e = hipEventElapsedTime(&kernel_ms[i], kt[i].start, kt[i].stop);
+      if (e != hipSuccess) rc = hip_fail("hipEventElapsedTime (kernel)", e);
+    }
   }
-  for (int i = 0; i <= MI_MOE_N_STAGES; ++i) (void)hipEventDestroy(ev[i]);
+  for (int i = 0; i < kEvents; ++i) (void)hipEventDestroy(ev[i]);
   return rc;
 } MI_CATCH("forward_timed")
 

@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 namespace mi_moe {
@@ -174,6 +175,26 @@ __device__ __forceinline__ T load_agent(const T *p) {
 template <class T>
 __device__ __forceinline__ void store_agent(T *p, T v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---------------------------------------------------------------- kernel timing (measurement only)
+// While a timer is installed on the calling thread (mi_moe_forward_timed does that), a grouped-product
+// launch goes through hipExtLaunchKernelGGL with the timer's two events: they then carry the start
+// and end time stamps of that dispatch itself, which is what a profiler reports as the kernel's
+// duration (an event recorded before and after a launch measures several microseconds more).
+struct KernelTimer {
+  hipEvent_t start = nullptr, stop = nullptr;
+  bool used = false;  // a kernel was launched with these events
+};
+extern thread_local KernelTimer *g_kernel_timer;
+template <class Kernel, class... Args>
+inline void launch_kernel(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t st, Args... args) {
+  if (KernelTimer *t = g_kernel_timer) {
+    hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)lds, st, t->start, t->stop, 0, args...);
+    t->used = true;
+  } else {
+    kernel<<<grid, block, lds, st>>>(args...);
+  }
 }
 
 // ---------------------------------------------------------------- launchers (host)

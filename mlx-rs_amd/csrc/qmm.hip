@@ -17,6 +17,8 @@
 
 namespace mi_moe {
 
+thread_local KernelTimer *g_kernel_timer = nullptr;
+
 __device__ __forceinline__ f32x4_t mfma16(const uint32_t (&a)[4], const uint32_t (&b)[4],
                                           f32x4_t c) {
   typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
@@ -756,7 +758,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
 #define MI_SMALL_LAUNCH(KWV, PR, SL, TGV, DV)                                                    \
   do {                                                                                         \
     if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV>), lds)) return; \
-    qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV><<<grid, 256, lds, st>>>(a, tt, sk);      \
+    launch_kernel(qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV>, grid, dim3(256), lds, st, a, tt, sk); \
   } while (0)
 #define MI_SMALL(KWV, TGV)                                                                     \
   do {                                                                                         \
@@ -772,7 +774,7 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
 #define MI_PAIR_LAUNCH(PR, TGV, DV)                                                              \
   do {                                                                                         \
     if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, false, 1, PR, false, TGV, DV, true>), lds)) return; \
-    qmm_small_kernel<BITS, false, 1, PR, false, TGV, DV, true><<<grid, 256, lds, st>>>(a, tt, sk); \
+    launch_kernel(qmm_small_kernel<BITS, false, 1, PR, false, TGV, DV, true>, grid, dim3(256), lds, st, a, tt, sk); \
   } while (0)
       if constexpr (BITS == 4) {
         if (two_groups) {

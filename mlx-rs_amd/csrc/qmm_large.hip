@@ -430,7 +430,8 @@ static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int li
       return e;
     if (dev >= 0 && dev < kMaxDevices) raised[dev].store(true, std::memory_order_release);
   }
-  qmm_large_kernel<BITS, GLU, MT><<<grid, NTHREADS, lds, st>>>(a, tiles, n_ntiles, list_cap, chunk, sub_log2);
+  launch_kernel(qmm_large_kernel<BITS, GLU, MT>, dim3(grid), dim3(NTHREADS), lds, st, a, tiles, n_ntiles, list_cap, chunk,
+                sub_log2);
   return hipGetLastError();
 }
 

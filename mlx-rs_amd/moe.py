@@ -127,8 +127,9 @@ class SparseMoeBlock:
 
     __call__ = forward
 
-    def forward_timed(self, x, out=None):
-        """One forward with HIP events between the stages; returns (out, stage_ms list)."""
+    def forward_timed(self, x, out=None, kernels=False):
+        """One forward with HIP events between the stages; returns (out, stage_ms list) and, with
+        kernels=True, the grouped-product kernels' own durations (capi.KERNEL_NAMES) as well."""
         _need(x, torch.bfloat16, "x")
         x2 = x.reshape(-1, self.config.hidden)
         T = x2.shape[0]
@@ -136,6 +137,9 @@ class SparseMoeBlock:
             out = torch.empty_like(x2)
         ws = self.reserve(max(T, 1))
         ms = (C.c_float * capi.N_STAGES)()
+        kms = (C.c_float * capi.N_KERNEL_TIMES)()
         check(self._lib.mi_moe_forward_timed(self._handle, _ptr(x2), T, _ptr(out), _ptr(ws), ws.numel(),
-                                             _stream(), ms))
+                                             _stream(), ms, kms))
+        if kernels:
+            return out.reshape(x.shape), list(ms), list(kms)
         return out.reshape(x.shape), list(ms)

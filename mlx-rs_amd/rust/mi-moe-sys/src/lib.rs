@@ -14,6 +14,7 @@ pub const MI_MOE_SCORE_SOFTMAX_THEN_TOPK_RENORM: i32 = 0;
 pub const MI_MOE_SCORE_SOFTMAX_THEN_TOPK: i32 = 1;
 pub const MI_MOE_SCORE_TOPK_THEN_SOFTMAX: i32 = 2;
 pub const MI_MOE_N_STAGES: usize = 6;
+pub const MI_MOE_N_KERNEL_TIMES: usize = 8;
 
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
@@ -69,7 +70,7 @@ extern "C" {
     pub fn mi_moe_forward(h: mi_moe_handle, x: *const u16, T: i64, out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, dbg: *const mi_moe_debug_out, stream: *mut c_void) -> c_int;
     pub fn mi_moe_forward_residual(h: mi_moe_handle, x: *const u16, norm_weight: *const u16, eps: f32, T: i64, out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, dbg: *const mi_moe_debug_out, stream: *mut c_void) -> c_int;
     pub fn mi_moe_rms_norm(x: *const u16, weight: *const u16, eps: f32, T: i64, hidden: i32, out: *mut u16, stream: *mut c_void) -> c_int;
-    pub fn mi_moe_forward_timed(h: mi_moe_handle, x: *const u16, T: i64, out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void, stage_ms: *mut f32) -> c_int;
+    pub fn mi_moe_forward_timed(h: mi_moe_handle, x: *const u16, T: i64, out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void, stage_ms: *mut f32, kernel_ms: *mut f32) -> c_int;
 
     pub fn mi_moe_route_workspace_size(n_experts: i32, T: i64, bytes: *mut usize) -> c_int;
     pub fn mi_moe_route(x: *const u16, router_w: *const u16, router_bias: *const f32, T: i64, hidden: i32, n_experts: i32, top_k: i32, score_mode: i32, topk_idx: *mut u32, topk_w: *mut u16, logits_out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;

@@ -66,7 +66,7 @@ def parse_header():
                 fields.append((nm.strip(), ty))
         structs[m.group(2)] = fields
     consts = {m.group(1): int(m.group(2)) for m in re.finditer(r"(MI_MOE_SCORE_\w+)\s*=\s*(\d+)", src)}
-    consts.update({m.group(1): int(m.group(2)) for m in re.finditer(r"#define\s+(MI_MOE_N_STAGES)\s+(\d+)", src)})
+    consts.update({m.group(1): int(m.group(2)) for m in re.finditer(r"#define\s+(MI_MOE_N_STAGES|MI_MOE_N_KERNEL_TIMES)\s+(\d+)", src)})
     return funcs, structs, consts
 
 
@@ -112,7 +112,7 @@ def test_structs_have_the_same_fields_in_the_same_order():
 def test_constants_agree():
     _, _, hc = parse_header()
     _, _, rc = parse_rust()
-    assert len(hc) == 4
+    assert len(hc) == 5
     assert hc == rc
 
 

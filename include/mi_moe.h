@@ -110,6 +110,21 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
                    void *workspace, size_t workspace_bytes, const mi_moe_debug_out *dbg,
                    void *stream);
 
+/* mi_moe_forward for callers that cannot allocate device memory or hand one over: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference (MLX allocates as it evaluates).  The workspace is an array of
+ * MI_MOE_STATIC_SCRATCH_BYTES that is part of the library's code object (each GPU the library runs on
+ * holds its own copy until the process ends); the call allocates nothing, creates nothing and gives
+ * mi_moe_forward's results bit for bit.  It fails, with a message that says how much is missing, when
+ * T tokens of the handle's layer need more workspace than that (mi_moe_workspace_size tells: the
+ * Qwen3-30B-A3B-shaped layer fits up to 156 tokens, the Mixtral-8x7B-shaped one up to 102, the
+ * Qwen3-235B-A22B-shaped one up to 84).  Every call on
+ * one GPU uses the same array, whatever the handle: calls that overlap on a GPU race, so keep them
+ * on one stream (or order them by events); nothing in the array has to survive between calls. */
+#define MI_MOE_STATIC_SCRATCH_BYTES 8388608
+int mi_moe_forward_static(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
+                          const mi_moe_debug_out *dbg, void *stream);
+
 /* The block between its neighbours in a decoder layer (mlx-lm/src/models/qwen3.rs:310-325:
  * r = post_attention_layernorm(h); r = mlp(r); out = h + r): out = x + moe(rms_norm(x, norm_weight,
  * eps)), with the residual add folded into the combine (one rounding) and the normalised rows

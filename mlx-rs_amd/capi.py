@@ -12,12 +12,13 @@ N_STAGES = 6
 N_KERNEL_TIMES = 8
 KERNEL_NAMES = ("gate_up_tiles256", "gate_up_tiles128", "gate_up_tiles64", "gate_up_streamed",
                 "down_tiles256", "down_tiles128", "down_tiles64", "down_streamed")
+STATIC_SCRATCH_BYTES = 8388608
 STAGE_NAMES = ("router_logits", "router_select", "dispatch", "gate_up_swiglu", "down", "combine")
 
 # every symbol include/mi_moe.h declares
 EXPORTS = (
     "mi_moe_last_error", "mi_moe_set_error_handler", "mi_moe_version", "mi_moe_create",
-    "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_forward_residual",
+    "mi_moe_destroy", "mi_moe_workspace_size", "mi_moe_forward", "mi_moe_forward_static", "mi_moe_forward_residual",
     "mi_moe_rms_norm", "mi_moe_forward_timed",
     "mi_moe_route_workspace_size",
     "mi_moe_route", "mi_moe_dispatch_workspace_size", "mi_moe_dispatch",
@@ -87,6 +88,7 @@ def load_library():
         "mi_moe_destroy": [vp],
         "mi_moe_workspace_size": [C.POINTER(Config), i64, C.POINTER(sz)],
         "mi_moe_forward": [vp, vp, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
+        "mi_moe_forward_static": [vp, vp, i64, vp, C.POINTER(DebugOut), vp],
         "mi_moe_forward_timed": [vp, vp, i64, vp, vp, sz, vp, C.POINTER(C.c_float), C.POINTER(C.c_float)],
         "mi_moe_forward_residual": [vp, vp, vp, C.c_float, i64, vp, vp, sz, C.POINTER(DebugOut), vp],
         "mi_moe_rms_norm": [vp, vp, C.c_float, i64, i32, vp, vp],

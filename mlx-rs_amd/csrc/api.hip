@@ -154,9 +154,16 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
 
 }  // namespace
 
+// Scratch of mi_moe_forward_static: the workspace a forward needs, as one array that is part of the
+// library's code object.  Every GPU that loads the library holds its own copy at its own address until
+// the process ends.  In host code the name is only a handle for hipGetSymbolAddress: the address a
+// kernel may use is looked up once per handle (mi_moe_create, on the handle's device) and kept there.
+static __device__ __align__(256) unsigned char scratch[MI_MOE_STATIC_SCRATCH_BYTES];
+
 struct mi_moe_s {
   mi_moe_config cfg;
   mi_moe_weights w;
+  unsigned char *scratch_dev = nullptr;  // device address of `scratch` on the handle's GPU
   uint32_t *counters = nullptr;  // device: arrival counters of the fused decode router, zero at rest
   // prefill-sized batches: the tile classes and the streamed segments are independent chains
   // (gate/up then down over the same rows); three of the four run on these streams, forked from
@@ -220,6 +227,9 @@ int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_mo
   }
   if (e == hipSuccess) e = hipEventCreateWithFlags(&h->fork, hipEventDisableTiming);
   if (e == hipSuccess) e = hipEventCreateWithFlags(&h->paired, hipEventDisableTiming);
+  // where the built-in scratch of mi_moe_forward_static lives on this GPU
+  if (e == hipSuccess) e = hipGetSymbolAddress(reinterpret_cast<void **>(&h->scratch_dev), HIP_SYMBOL(scratch));
+  if (e == hipSuccess && (!h->scratch_dev || (reinterpret_cast<uintptr_t>(h->scratch_dev) & 255u))) e = hipErrorInvalidSymbol;
   if (e != hipSuccess) {
     destroy_handle(h);
     return fail("create: device memory, streams and events of the handle: %s", hipGetErrorString(e));
@@ -453,6 +463,21 @@ int mi_moe_forward(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
                    size_t workspace_bytes, const mi_moe_debug_out *dbg, void *stream) try {
   return forward_impl(h, x, T, out, workspace, workspace_bytes, dbg, static_cast<hipStream_t>(stream), nullptr);
 } MI_CATCH("forward")
+
+int mi_moe_forward_static(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out,
+                          const mi_moe_debug_out *dbg, void *stream) try {
+  if (!h) return fail("forward_static: handle is NULL");
+  if (T < 0) return fail("forward_static: negative token count");
+  if (T * (int64_t)h->cfg.top_k > (int64_t)1 << 30) return fail("forward_static: too many (token, expert) pairs");
+  const size_t need = carve_forward(h->cfg, T, nullptr).bytes;
+  if (need > (size_t)MI_MOE_STATIC_SCRATCH_BYTES)
+    return fail("forward_static: %lld tokens of this layer need %zu bytes of workspace, the built-in scratch holds %zu "
+                "(use mi_moe_forward with a workspace of the caller's)",
+                (long long)T, need, (size_t)MI_MOE_STATIC_SCRATCH_BYTES);
+  // no allocation from here on: the kernels get the address looked up by mi_moe_create
+  return forward_impl(h, x, T, out, h->scratch_dev, (size_t)MI_MOE_STATIC_SCRATCH_BYTES, dbg,
+                      static_cast<hipStream_t>(stream), nullptr);
+} MI_CATCH("forward_static")
 
 int mi_moe_forward_residual(mi_moe_handle h, const uint16_t *x, const uint16_t *norm_weight, float eps,
                             int64_t T, uint16_t *out, void *workspace, size_t workspace_bytes,

@@ -90,6 +90,20 @@ class SparseMoeBlock:
         the residual add behind it (mlx-lm/src/models/qwen3.rs:310-325) in one call."""
         return self.forward(x, debug=debug, out=out, _norm=(_need(norm_weight, torch.bfloat16, "norm_weight"), eps))
 
+    def forward_static(self, x, out=None):
+        """forward() on the library's built-in scratch instead of a workspace tensor
+        (mi_moe_forward_static): nothing is allocated by the call when ``out`` is given.  Raises
+        when the batch needs more workspace than the scratch holds."""
+        _need(x, torch.bfloat16, "x")
+        c = self.config
+        if x.shape[-1] != c.hidden:
+            raise capi.MoeError(f"forward_static: last dimension must be {c.hidden}, got {x.shape[-1]}")
+        x2 = x.reshape(-1, c.hidden)
+        if out is None:
+            out = torch.empty_like(x2)
+        check(self._lib.mi_moe_forward_static(self._handle, _ptr(x2), x2.shape[0], _ptr(out), None, _stream()))
+        return out.reshape(x.shape)
+
     def forward(self, x, debug=False, out=None, _norm=None):
         """x: bf16 [..., H] -> bf16 [..., H].  With debug=True also returns the routing
         arrays (topk_idx, topk_w, counts, offsets, perm, inv_perm)."""

@@ -15,6 +15,7 @@ pub const MI_MOE_SCORE_SOFTMAX_THEN_TOPK: i32 = 1;
 pub const MI_MOE_SCORE_TOPK_THEN_SOFTMAX: i32 = 2;
 pub const MI_MOE_N_STAGES: usize = 6;
 pub const MI_MOE_N_KERNEL_TIMES: usize = 8;
+pub const MI_MOE_STATIC_SCRATCH_BYTES: usize = 8388608;
 
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
@@ -68,6 +69,7 @@ extern "C" {
     pub fn mi_moe_destroy(h: mi_moe_handle) -> c_int;
     pub fn mi_moe_workspace_size(cfg: *const mi_moe_config, max_tokens: i64, bytes: *mut usize) -> c_int;
     pub fn mi_moe_forward(h: mi_moe_handle, x: *const u16, T: i64, out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, dbg: *const mi_moe_debug_out, stream: *mut c_void) -> c_int;
+    pub fn mi_moe_forward_static(h: mi_moe_handle, x: *const u16, T: i64, out: *mut u16, dbg: *const mi_moe_debug_out, stream: *mut c_void) -> c_int;
     pub fn mi_moe_forward_residual(h: mi_moe_handle, x: *const u16, norm_weight: *const u16, eps: f32, T: i64, out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, dbg: *const mi_moe_debug_out, stream: *mut c_void) -> c_int;
     pub fn mi_moe_rms_norm(x: *const u16, weight: *const u16, eps: f32, T: i64, hidden: i32, out: *mut u16, stream: *mut c_void) -> c_int;
     pub fn mi_moe_forward_timed(h: mi_moe_handle, x: *const u16, T: i64, out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void, stage_ms: *mut f32, kernel_ms: *mut f32) -> c_int;

@@ -1,15 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized MoE layer on one MI355X.
 
-Default workload = the Qwen3-30B-A3B-shaped layer at decode (hidden 2048, 128 experts,
-top-8 renormalised, intermediate 768, 4-bit g64), batches 1 / 8 / 32; the headline
-`value` is tokens/s at batch 32.  A "step" is one forward of the layer over one batch
-whose inputs are already in HBM.  Steps rotate over several distinct weight sets whose
-total size exceeds the 256 MB Infinity Cache, so weights stream from HBM every step.
+The default run measures both halves of the metric on the Qwen3-30B-A3B-shaped layer (hidden 2048,
+128 experts, top-8 renormalised, intermediate 768, 4-bit g64):
+  * decode, batches 1 / 8 / 32 -- the headline `value` is tokens/s at batch 32, `roofline` prices the
+    dominant kernel of that step against the HBM peak;
+  * prefill, 4096 tokens with a Zipf(1.1) router bias -- `roofline_prefill` prices its dominant kernel
+    against the dense bf16 MFMA peak, `prefill` holds tokens/s and the layer-level fraction.
+A "step" is one forward of the layer over one batch whose inputs are already in HBM.  Steps rotate
+over several distinct weight sets whose total size exceeds the 256 MB Infinity Cache, so weights
+stream from HBM every step.
 
-Prints ONE JSON line (see --help for the other workloads).  The CPU-baseline leg times
-the CPU oracle (a restatement of the MLX CPU op sequence; MLX itself is not available)
-on the host cores; it is the only part of this script that touches oracle/.
+Kernel durations are the ones mi_moe_forward_timed reports from each dispatch's own start and end
+time stamps (what rocprofv3 lists as the kernel's duration), averaged over the timed steps.
+
+Prints ONE JSON line (see --help for the other workloads).  The CPU-baseline leg times the CPU
+oracle (a restatement of the MLX CPU op sequence; MLX itself is not available) on the host cores;
+it is the only part of this script that touches oracle/.
 """
 import argparse
 import json
@@ -22,12 +29,24 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
-# HBM bytes per launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE scaled by
-# what the same counters read for a plain copy kernel (profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt,
-# profiles/qmm_small_kernel_decode_mixtral_batch1.txt,
-# profiles/qmm_large_kernel_prefill_tokens4096_counters.txt);
-# counters cannot be read from inside this script, so the figure is carried here per workload.
-MEASURED_TRAFFIC_BYTES = {"decode": 1.976e8, "prefill": 5.50e8, "mixtral_decode": 2.530e8}
+# HBM bytes per launch of each workload's roofline kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
+# scaled by what the same counters read for a plain copy kernel of known size.  Counters cannot be read from
+# inside this script: the figure is carried from the named file under profiles/, it is not measured by this run.
+CARRIED_TRAFFIC = {
+    "decode": (1.976e8, "profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt"),
+    "prefill": (5.50e8, "profiles/qmm_large_kernel_prefill_tokens4096_counters.txt"),
+    "mixtral_decode": (2.530e8, "profiles/qmm_small_kernel_decode_mixtral_batch1.txt"),
+}
+
+WORKLOADS = {
+    # name: (config key, batches, headline batch, zipf s, bound)
+    "decode": ("qwen3_30b_a3b", [1, 8, 32], 32, None, "hbm"),
+    "prefill": ("qwen3_30b_a3b", [4096], 4096, 1.1, "mfma"),
+    "mixtral_decode": ("mixtral_8x7b", [1], 1, None, "hbm"),
+    "mixtral_prefill": ("mixtral_8x7b", [2048], 2048, None, "mfma"),
+    "qwen3_235b_prefill": ("qwen3_235b_a22b", [8192], 8192, 1.3, "mfma"),
+    "tiny": ("tiny", [32], 32, None, "hbm"),
+}
 
 
 def parse():
@@ -35,8 +54,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="decode",
-                    choices=["decode", "prefill", "mixtral_decode", "mixtral_prefill", "qwen3_235b_prefill", "tiny"])
+    ap.add_argument("--workload", default="default", choices=["default"] + sorted(WORKLOADS),
+                    help="default = decode (headline) followed by prefill, both in the one JSON line")
     ap.add_argument("--layers", type=int, default=0, help="distinct weight sets to rotate over (0 = auto)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
@@ -51,17 +70,6 @@ def parse():
     return ap.parse_args()
 
 
-WORKLOADS = {
-    # name: (config key, batches, headline batch, zipf s, bound)
-    "decode": ("qwen3_30b_a3b", [1, 8, 32], 32, None, "hbm"),
-    "prefill": ("qwen3_30b_a3b", [4096], 4096, 1.1, "mfma"),
-    "mixtral_decode": ("mixtral_8x7b", [1], 1, None, "hbm"),
-    "mixtral_prefill": ("mixtral_8x7b", [2048], 2048, None, "mfma"),
-    "qwen3_235b_prefill": ("qwen3_235b_a22b", [8192], 8192, 1.3, "mfma"),
-    "tiny": ("tiny", [32], 32, None, "hbm"),
-}
-
-
 def time_steps(fn, steps, warmup, torch):
     for i in range(warmup):
         fn(i)
@@ -73,39 +81,49 @@ def time_steps(fn, steps, warmup, torch):
     return (time.perf_counter() - t0) / steps * 1e3
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
-              file=sys.stderr)
-        sys.exit(2)
-    import torch
-    import mlx_rs_amd as m
-    from mlx_rs_amd import synth
+def tile_class_rows(counts, cfg, T):
+    """Rows of the batch that each grouped-product kernel processes: [256-row tiles, 128-row tiles,
+    64-row tiles, streamed], by the library's rule (segments of tmr rows and more are cut into 256-row
+    tiles, the remainder goes to the smallest class that holds it; shorter segments stream)."""
+    P, E = T * cfg.top_k, cfg.n_experts
+    light, heavy_avg = (6, 20) if cfg.bits == 4 else (17, 17)
+    even_groups = (cfg.hidden // 64) % 2 == 0 and (cfg.intermediate // 64) % 2 == 0
+    heavy = P >= heavy_avg * E
+    tiled = even_groups and (P >= light * E or heavy)
+    tmr = (9 if heavy else 17) if cfg.bits == 4 else 17
+    rows = [0, 0, 0, 0]
+    for c in counts:
+        c = int(c)
+        if not tiled or c < tmr:
+            rows[3] += c
+            continue
+        full, r = divmod(c, 256)
+        rows[0] += full * 256
+        if r > 128:
+            rows[0] += r
+        elif r > 64:
+            rows[1] += r
+        else:
+            rows[2] += r
+    return rows
 
-    m.load_library()  # raises if the HIP library is missing
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    dev = "cuda:0"
-    torch.cuda.set_device(0)
-    cfg_name, batches, headline, zipf_s, bound = WORKLOADS[args.workload]
+
+def run_workload(name, args, torch, m, synth, dev):
+    """Times one workload; returns a dict with the headline step, the per-batch detail and what the
+    roofline block needs."""
+    cfg_name, batches, headline, zipf_s, bound = WORKLOADS[name]
     if args.only_headline:
         batches = [headline]
-    if args.batches:
+    if args.batches and args.workload != "default":
         batches = sorted(set(int(b) for b in args.batches.split(",")) | {headline})
-    if args.copy_probe:
-        # an elementwise kernel that reads 256 MiB and writes 256 MiB
-        src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(args.copy_probe):
-            torch.add(src, 1, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
     cfg = synth.CONFIGS[cfg_name]
-    per_expert = synth.layer_bytes_per_expert(cfg)
-    layer_bytes = per_expert * cfg.n_experts
+    layer_bytes = synth.layer_bytes_per_expert(cfg) * cfg.n_experts
     n_layers = args.layers or max(2, min(8, int(1.4e9 // layer_bytes) + 1))
     if layer_bytes > 1.0e9:
         n_layers = args.layers or 2
+    steps, warmup = args.steps, args.warmup
+    if bound == "mfma" and args.workload == "default":
+        steps, warmup = max(10, steps // 4), max(2, warmup // 4)  # a prefill step is 7 times a decode step
     blocks = [synth.make_block(cfg, seed=args.seed + 31 * i, device=dev, zipf_s=zipf_s, gen_device="cuda")
               for i in range(n_layers)]
     torch.cuda.synchronize()
@@ -118,13 +136,15 @@ def main():
         for b in blocks:
             b.reserve(T)
         # realised routing (per weight set)
-        actives, counts_stats = [], []
+        actives, counts_stats, class_rows = [], [], []
         for b in blocks:
             _, dbg = b.forward(x, debug=True)
             c = dbg["counts"].cpu().numpy()
             actives.append(int((c > 0).sum()))
             counts_stats.append((int(c.max()), float(c.mean()), int(c.min())))
+            class_rows.append(tile_class_rows(c, cfg, T))
         n_active = sum(actives) / len(actives)
+        class_rows = [sum(r[i] for r in class_rows) / len(class_rows) for i in range(4)]
 
         if args.serial_kernels:
             step_fn = lambda blk, xx, oo: blk.forward_timed(xx, out=oo)
@@ -153,20 +173,18 @@ def main():
 
         if graph is not None:
             # a step = one forward; one replay = n_layers steps
-            reps = max(1, args.steps // n_layers)
-            wreps = max(1, args.warmup // n_layers)
+            reps = max(1, steps // n_layers)
+            wreps = max(1, warmup // n_layers)
             ms = time_steps(lambda i: graph.replay(), reps, wreps, torch) / n_layers
             steps_done = reps * n_layers
         else:
-            ms = time_steps(lambda i: step_fn(blocks[i % n_layers], x, outs[i % n_layers]),
-                            args.steps, args.warmup, torch)
-            steps_done = args.steps
-        eager_ms = time_steps(lambda i: step_fn(blocks[i % n_layers], x, outs[i % n_layers]),
-                              args.steps, args.warmup, torch)
+            ms = time_steps(lambda i: step_fn(blocks[i % n_layers], x, outs[i % n_layers]), steps, warmup, torch)
+            steps_done = steps
+        eager_ms = time_steps(lambda i: step_fn(blocks[i % n_layers], x, outs[i % n_layers]), steps, warmup, torch)
 
         # spread of single steps (event pair around each eager step) and the cache-resident figure
         # (one weight set only: at decode sizes it stays in the 256 MB Infinity Cache)
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         for i, (e0, e1) in enumerate(evs):
             e0.record()
             step_fn(blocks[i % n_layers], x, outs[i % n_layers])
@@ -174,14 +192,18 @@ def main():
         torch.cuda.synchronize()
         per_step = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
         pct = lambda q: per_step[min(len(per_step) - 1, int(q * len(per_step)))]
-        resident_ms = time_steps(lambda i: step_fn(blocks[0], x, outs[0]), args.steps, args.warmup, torch)
+        resident_ms = time_steps(lambda i: step_fn(blocks[0], x, outs[0]), steps, warmup, torch)
 
-        # per-kernel durations from HIP events on the launch stream, same K steps
+        # per-stage times (events between the stages) and the grouped-product kernels' own durations
+        # (time stamps of each dispatch), same number of steps
         stage = [0.0] * m.capi.N_STAGES
-        for i in range(args.steps):
-            _, st = blocks[i % n_layers].forward_timed(x, out=outs[i % n_layers])
+        kern = [0.0] * m.capi.N_KERNEL_TIMES
+        for i in range(steps):
+            _, st, km = blocks[i % n_layers].forward_timed(x, out=outs[i % n_layers], kernels=True)
             stage = [a + b for a, b in zip(stage, st)]
-        stage = [v / args.steps for v in stage]
+            kern = [a + b for a, b in zip(kern, km)]
+        stage = [v / steps for v in stage]
+        kern = [v / steps for v in kern]
 
         P = T * cfg.top_k
         qbytes = lambda n, k: n * k * cfg.bits // 8 + (n * k // cfg.group_size) * 4
@@ -190,6 +212,7 @@ def main():
         alg_bytes = synth.decode_algorithmic_bytes(cfg, T, n_active)
         flops = synth.prefill_flops(cfg, T)
         gu_flops = P * 2 * 2 * cfg.hidden * cfg.intermediate
+        gu_kernel_ms, dn_kernel_ms = sum(kern[0:4]), sum(kern[4:8])
         detail[str(T)] = {
             "tokens_per_s": T / (ms * 1e-3), "ms_per_step": ms, "ms_per_step_eager": eager_ms,
             "steps": steps_done, "active_experts": n_active,
@@ -200,58 +223,104 @@ def main():
             "layer_hbm_frac": alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "layer_TFLOPs": flops / (ms * 1e-3) / 1e12,
             "layer_mfma_frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-            "stage_us": {n: round(v * 1e3, 2) for n, v in zip(m.capi.STAGE_NAMES, stage)},
-            "gate_up_GBps": gu_bytes / (stage[3] * 1e-3) / 1e9,
-            "down_GBps": dn_bytes / (stage[4] * 1e-3) / 1e9,
-            "gate_up_TFLOPs": gu_flops / (stage[3] * 1e-3) / 1e12,
+            "stage_us_between_events": {n: round(v * 1e3, 2) for n, v in zip(m.capi.STAGE_NAMES, stage)},
+            "kernel_us": {n: round(v * 1e3, 2) for n, v in zip(m.capi.KERNEL_NAMES, kern) if v > 0},
+            "rows_per_kernel_class": dict(zip(("tiles256", "tiles128", "tiles64", "streamed"), class_rows)),
+            "gate_up_GBps": gu_bytes / (gu_kernel_ms * 1e-3) / 1e9 if gu_kernel_ms else None,
+            "down_GBps": dn_bytes / (dn_kernel_ms * 1e-3) / 1e9 if dn_kernel_ms else None,
+            "gate_up_TFLOPs": gu_flops / (gu_kernel_ms * 1e-3) / 1e12 if gu_kernel_ms else None,
+            "gate_up_mfma_frac": gu_flops / (gu_kernel_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS if gu_kernel_ms else None,
         }
         if T == headline:
-            head = dict(ms=ms, T=T, gu_bytes=gu_bytes, gu_ms=stage[3], gu_flops=gu_flops, steps=steps_done)
-            # What a pair of timed events adds around a kernel: the same pair with nothing in between,
-            # on the same stream (median of 200).  The stage time minus this is what rocprofv3 reports
-            # as the kernel's own duration.
-            pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(200)]
-            for e0, e1 in pairs:
-                e0.record()
-                e1.record()
-            torch.cuda.synchronize()
-            empty = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
-            head["pair_ms"] = min(empty[len(empty) // 2], 0.5 * stage[3])
+            head = dict(ms=ms, T=T, gu_bytes=gu_bytes, dn_bytes=dn_bytes, gu_flops=gu_flops, steps=steps_done, warmup=warmup, kern=kern,
+                        class_rows=class_rows, per_row_gu_flops=2 * 2 * cfg.hidden * cfg.intermediate)
         del outs, graph
 
-    kernel_ms = head["gu_ms"] - head["pair_ms"]
-    timing = {"kernel_us": kernel_ms * 1e3, "kernel_us_between_events": head["gu_ms"] * 1e3,
-              "empty_event_pair_us": head["pair_ms"] * 1e3}
+    traffic, traffic_src = CARRIED_TRAFFIC.get(name, (None, None))
     if bound == "hbm":
-        achieved = head["gu_bytes"] / (kernel_ms * 1e-3) / 1e9
-        roofline = {"kernel": "qmm_small_kernel (gate/up + SwiGLU)", "bound": "hbm", "achieved": achieved,
+        # the streamed gate/up + SwiGLU kernel: every segment streams at decode sizes
+        k_ms, k_bytes = head["kern"][3], head["gu_bytes"]
+        k_name = "qmm_small_kernel (gate/up + SwiGLU, streamed)"
+        achieved = k_bytes / (k_ms * 1e-3) / 1e9
+        roofline = {"kernel": k_name, "bound": "hbm", "achieved": achieved,
                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                    "algorithmic_bytes_per_launch": head["gu_bytes"], **timing,
+                    "traffic": traffic, "traffic_source": traffic_src and traffic_src + " (carried, not measured by this run)",
+                    "algorithmic_bytes_per_launch": head["gu_bytes"], "kernel_us": k_ms * 1e3,
+                    "kernel_us_source": "start/end time stamps of the dispatch (hipExtLaunchKernelGGL events), mean over the timed steps",
                     "stream_probe": stream_probe(m, head["gu_bytes"], dev)}
     else:
-        achieved = head["gu_flops"] / (kernel_ms * 1e-3) / 1e12
-        roofline = {"kernel": "grouped qmm (gate/up + SwiGLU)", "bound": "mfma", "achieved": achieved,
-                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                    "algorithmic_flops_per_launch": head["gu_flops"], **timing}
+        # the dominant kernel: the tile class that holds most rows (256-row tiles at prefill sizes)
+        cls = max(range(3), key=lambda i: head["class_rows"][i])
+        k_ms, k_rows = head["kern"][cls], head["class_rows"][cls]
+        k_name = "qmm_large_kernel (gate/up + SwiGLU, %d-row tiles)" % (256, 128, 64)[cls]
+        k_flops = k_rows * head["per_row_gu_flops"]
+        achieved = k_flops / (k_ms * 1e-3) / 1e12
+        roofline = {"kernel": k_name, "bound": "mfma",
+                    "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                    "traffic": traffic, "traffic_source": traffic_src and traffic_src + " (carried, not measured by this run)",
+                    "algorithmic_flops_per_launch": k_flops, "rows_per_launch": k_rows,
+                    "kernel_us": k_ms * 1e3,
+                    "kernel_us_source": "start/end time stamps of the dispatch (hipExtLaunchKernelGGL events), mean over the timed steps",
+                    "gate_up_stage": {"flops": head["gu_flops"], "kernels_us": sum(head["kern"][0:4]) * 1e3,
+                                      "TFLOPs": head["gu_flops"] / (sum(head["kern"][0:4]) * 1e-3) / 1e12,
+                                      "frac": head["gu_flops"] / (sum(head["kern"][0:4]) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS}}
+    workload = "%s %s-bit g64 MoE layer, %s, batch %d" % (cfg_name, cfg.bits, name, headline)
+    config = {"workload": workload, "hidden": cfg.hidden, "n_experts": cfg.n_experts, "top_k": cfg.top_k,
+              "intermediate": cfg.intermediate, "bits": cfg.bits, "batch": headline, "weight_sets_rotated": n_layers,
+              "zipf_s": zipf_s,
+              "launch": "eager, one kernel at a time" if args.serial_kernels else ("eager" if args.no_graph else "hip-graph")}
+    return dict(cfg=cfg, blocks=blocks, head=head, headline=headline, detail=detail, roofline=roofline, bound=bound,
+                config=config)
 
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import mlx_rs_amd as m
+    from mlx_rs_amd import synth
+
+    m.load_library()  # raises if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    if args.copy_probe:
+        # an elementwise kernel that reads 256 MiB and writes 256 MiB
+        src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.copy_probe):
+            torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
+    first = "decode" if args.workload == "default" else args.workload
+    w = run_workload(first, args, torch, m, synth, dev)
+    head, bound = w["head"], w["bound"]
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(cfg, blocks[0], headline, args.seed, synth)
-
+        cpu = cpu_baseline(w["cfg"], w["blocks"][0], w["headline"], args.seed, synth)
     out = {
         "metric": "MoE-layer tokens/sec (%s)" % ("decode" if bound == "hbm" else "prefill"),
-        "value": headline / (head["ms"] * 1e-3), "unit": "tokens/s", "n_gpus": 1,
-        "steps": head["steps"], "warmup": args.warmup, "ms_per_step": head["ms"],
+        "value": w["headline"] / (head["ms"] * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": head["steps"], "warmup": head["warmup"], "ms_per_step": head["ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": "%s %s-bit g64 MoE layer, %s, batch %d" % (cfg_name, cfg.bits, args.workload, headline),
-                   "hidden": cfg.hidden, "n_experts": cfg.n_experts, "top_k": cfg.top_k,
-                   "intermediate": cfg.intermediate, "bits": cfg.bits, "batch": headline,
-                   "weight_sets_rotated": n_layers, "launch": "eager, one kernel at a time" if args.serial_kernels else ("eager" if args.no_graph else "hip-graph")},
-        "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
+        "data": "synthetic", "config": w["config"],
+        "layer_frac_of_peak": w["detail"][str(w["headline"])]["layer_hbm_frac" if bound == "hbm" else "layer_mfma_frac"],
+        "roofline": w["roofline"], "cpu_baseline": cpu, "detail": w["detail"],
     }
+    if args.workload == "default":
+        del w  # the decode weight sets go before the prefill ones are built
+        torch.cuda.empty_cache()
+        p = run_workload("prefill", args, torch, m, synth, dev)
+        d = p["detail"][str(p["headline"])]
+        out["roofline_prefill"] = p["roofline"]
+        out["prefill"] = {"metric": "MoE-layer tokens/sec (prefill)", "value": d["tokens_per_s"], "unit": "tokens/s",
+                          "ms_per_step": d["ms_per_step"], "steps": d["steps"], "config": p["config"],
+                          "layer_TFLOPs": d["layer_TFLOPs"], "layer_frac_of_peak": d["layer_mfma_frac"], "detail": d}
     print(json.dumps(out))
 
 

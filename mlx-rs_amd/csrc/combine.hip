@@ -8,23 +8,39 @@
 
 namespace mi_moe {
 
-__global__ __launch_bounds__(256) void combine_kernel(
+// One thread per 8 output columns, kCombineThreads threads per block (a token's row is spread over
+// several blocks: at decode sizes the launch is latency, and a block per token would leave most of
+// the chip idle).  The k rows of a token are fetched eight at a time, all loads of a batch in flight
+// before the first is used; the sum itself runs in slot order.
+constexpr int kCombineThreads = 64;
+__global__ __launch_bounds__(kCombineThreads) void combine_kernel(
     const uint16_t *__restrict__ y, const uint16_t *__restrict__ scores,
     const uint32_t *__restrict__ inv_perm, int64_t T, int k, int H,
     const uint16_t *__restrict__ residual, uint16_t *__restrict__ out) {
   const int64_t t = blockIdx.x;
-  const int h = (blockIdx.y * 256 + threadIdx.x) * 8;
+  const int h = (blockIdx.y * kCombineThreads + threadIdx.x) * 8;
   if (h >= H) return;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < k; ++s) {
-    const int64_t r = inv_perm ? (int64_t)inv_perm[t * k + s] : t * k + s;
-    const float sc = bf16_to_f32(scores[t * k + s]);
-    const uint4 v = *reinterpret_cast<const uint4 *>(y + r * H + h);
-    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+  for (int s0 = 0; s0 < k; s0 += 8) {
+    uint4 v[8];
+    float sc[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      acc[2 * i] += sc * bf16lo_to_f32(u[i]);
-      acc[2 * i + 1] += sc * bf16hi_to_f32(u[i]);
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < k ? s0 + j : k - 1;  // (clamped: loads without a condition stay in flight together)
+      const int64_t r = inv_perm ? (int64_t)inv_perm[t * k + s] : t * k + s;
+      sc[j] = bf16_to_f32(scores[t * k + s]);
+      v[j] = *reinterpret_cast<const uint4 *>(y + r * H + h);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (s0 + j < k) {
+        const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc[2 * i] += sc[j] * bf16lo_to_f32(u[i]);
+          acc[2 * i + 1] += sc[j] * bf16hi_to_f32(u[i]);
+        }
+      }
     }
   }
   if (residual) {  // h + mlp(...): the block's neighbour in a decoder layer, added before the one rounding
@@ -48,8 +64,8 @@ hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint3
                           int64_t T, int k, int H, const uint16_t *residual, uint16_t *out,
                           hipStream_t st) {
   if (T == 0) return hipSuccess;
-  dim3 grid((unsigned)T, (unsigned)((H / 8 + 255) / 256));
-  combine_kernel<<<grid, 256, 0, st>>>(y, scores, inv_perm, T, k, H, residual, out);
+  dim3 grid((unsigned)T, (unsigned)((H / 8 + kCombineThreads - 1) / kCombineThreads));
+  combine_kernel<<<grid, kCombineThreads, 0, st>>>(y, scores, inv_perm, T, k, H, residual, out);
   return hipGetLastError();
 }
 

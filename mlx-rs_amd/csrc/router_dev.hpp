@@ -11,14 +11,28 @@ namespace mi_moe {
 __device__ __forceinline__ double logit_wave(const uint16_t *__restrict__ xr,
                                              const uint16_t *__restrict__ wr, int H) {
   double acc = 0.0;
-  for (int h = lane_id() * 8; h < H; h += kWave * 8) {
-    const uint4 xv = *reinterpret_cast<const uint4 *>(xr + h);
-    const uint4 wv = *reinterpret_cast<const uint4 *>(wr + h);
-    const uint32_t xu[4] = {xv.x, xv.y, xv.z, xv.w}, wu[4] = {wv.x, wv.y, wv.z, wv.w};
+  // four pieces of each row per pass, all eight loads in flight before the first is used (a pass
+  // covers 2048 values: one memory round trip for a row of that length instead of four); the
+  // additions keep the order of a plain loop over the pieces
+  for (int h0 = lane_id() * 8; h0 < H; h0 += 4 * kWave * 8) {
+    uint4 xv[4], wv[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      acc = __builtin_fma((double)bf16lo_to_f32(xu[q]), (double)bf16lo_to_f32(wu[q]), acc);
-      acc = __builtin_fma((double)bf16hi_to_f32(xu[q]), (double)bf16hi_to_f32(wu[q]), acc);
+    for (int p = 0; p < 4; ++p) {
+      const int h = h0 + p * kWave * 8;
+      const int hc = h < H ? h : h0;  // (clamped: the loads carry no condition)
+      xv[p] = *reinterpret_cast<const uint4 *>(xr + hc);
+      wv[p] = *reinterpret_cast<const uint4 *>(wr + hc);
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      if (h0 + p * kWave * 8 < H) {
+        const uint32_t xu[4] = {xv[p].x, xv[p].y, xv[p].z, xv[p].w}, wu[4] = {wv[p].x, wv[p].y, wv[p].z, wv[p].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc = __builtin_fma((double)bf16lo_to_f32(xu[q]), (double)bf16lo_to_f32(wu[q]), acc);
+          acc = __builtin_fma((double)bf16hi_to_f32(xu[q]), (double)bf16hi_to_f32(wu[q]), acc);
+        }
+      }
     }
   }
   return wave_sum_f64(acc);

@@ -56,13 +56,22 @@ typedef enum {
   MI_MOE_SCORE_TOPK_THEN_SOFTMAX = 2         /* Mixtral: softmax over the selected logits */
 } mi_moe_score_mode;
 
+/* element type of activations, scales, biases and outputs of the *_typed entry points (MLX takes
+ * any floating type there, mlx-rs/src/dtype.rs:206-256; the reference's own tests of these ops run in
+ * float32, mlx-rs/src/ops/quantization.rs:318-423) */
+typedef enum {
+  MI_MOE_DTYPE_BF16 = 0,
+  MI_MOE_DTYPE_F16 = 1,
+  MI_MOE_DTYPE_F32 = 2
+} mi_moe_dtype;
+
 typedef struct {
   int32_t hidden;       /* H, multiple of group_size */
   int32_t n_experts;    /* E, 1..512 */
   int32_t top_k;        /* k, 1..min(E,32) */
   int32_t intermediate; /* I, multiple of group_size */
-  int32_t bits;         /* 4 or 8 */
-  int32_t group_size;   /* 64 */
+  int32_t bits;         /* 4 or 8 (tuned kernels); 2 runs on the plain products */
+  int32_t group_size;   /* 64 (tuned kernels); 32 and 128 run on the plain products */
   int32_t score_mode;   /* mi_moe_score_mode */
 } mi_moe_config;
 
@@ -179,10 +188,14 @@ int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts
 /* ---- R6 gather_qmm (mlx_gather_qmm, mlx-rs/src/ops/quantization.rs:160-230):
  * for j < n_idx: y[j] (M x N) = x[lhs[j]] (M x K) . dequantize(w[rhs[j]])^T.
  * x: bf16 [x_batch, M, K]; w: [E, N, K*bits/32]; y: bf16 [n_idx, M, N].
- * lhs_indices NULL = identity (j), as an absent mlx_array; rhs_indices required.
- * transpose non-zero is the layout every mlx-lm switch layer uses and the tuned path; with
- * transpose = 0, w is [E, K, N*bits/32] with scales, biases [E, K, N/group_size] (K x N matrices
- * quantised along N, N a multiple of 64), served by a plain kernel that needs no workspace.
+ * lhs_indices NULL = identity (j), as an absent mlx_array; rhs_indices required.  Index arrays of
+ * other shapes are broadcast against each other and flattened by the host layers (the op's batch
+ * semantics, :160-176); the entry point takes the flat arrays.
+ * The tuned path: transpose non-zero (the layout every mlx-lm switch layer uses), group_size 64,
+ * bits 4 or 8, K a multiple of 64 (4-bit: 128), N a multiple of 16, at most 512 experts.  Everything
+ * else -- transpose = 0 (w [E, K, N*bits/32], scales, biases [E, K, N/group_size], K x N matrices
+ * quantised along N), group sizes 32 and 128, 2-bit codes -- is served by plain kernels that need no
+ * workspace and no alignment.
  * sorted_indices is a hint, results do not depend on it.
  * workspace >= mi_moe_gather_qmm_workspace_size. */
 int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M, size_t *bytes);
@@ -192,19 +205,35 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
                       int32_t N, int32_t K, int32_t n_experts, int32_t transpose,
                       int32_t group_size, int32_t bits, int32_t sorted_indices, uint16_t *y,
                       void *workspace, size_t workspace_bytes, void *stream);
+/* the same op with x, scales, biases and y of element type dtype (mi_moe_dtype); bf16 takes the
+ * paths above, fp16 and fp32 the plain kernels (fp32 accumulation, one rounding to dtype):
+ * test_gather_qmm of the reference (mlx-rs/src/ops/quantization.rs:345-423) runs through this. */
+int mi_moe_gather_qmm_typed(const void *x, const uint32_t *w, const void *scales, const void *biases,
+                            const uint32_t *lhs_indices, const uint32_t *rhs_indices, int64_t n_idx,
+                            int64_t x_batch, int32_t M, int32_t N, int32_t K, int32_t n_experts,
+                            int32_t transpose, int32_t group_size, int32_t bits,
+                            int32_t sorted_indices, int32_t dtype, void *y, void *workspace,
+                            size_t workspace_bytes, void *stream);
 
 /* ---- dense quantized matmul (mlx_quantized_matmul, mlx-rs/src/ops/quantization.rs:91-122, as
  * QuantizedLinear::forward calls it with transpose = true, mlx-rs/src/nn/quantized.rs:363-386):
  * y (M x N) = x (M x K) . dequantize(w)^T on the same kernels as gather_qmm (one matrix, every row).
  * x: bf16 [M, K]; w: [N, K*bits/32]; scales, biases: bf16 [N, K/group_size]; y: bf16 [M, N].
  * transpose = 0 (the op's own default; test_quantized_matmul, ops/quantization.rs:318-342):
- * w [K, N*bits/32], scales, biases [K, N/group_size], y = x . dequantize(w), a plain kernel.
- * workspace >= mi_moe_quantized_matmul_workspace_size (transpose = 0 needs none). */
+ * w [K, N*bits/32], scales, biases [K, N/group_size], y = x . dequantize(w), a plain kernel; so are
+ * group sizes 32 / 128 and 2-bit codes.
+ * workspace >= mi_moe_quantized_matmul_workspace_size (the plain kernels need none). */
 int mi_moe_quantized_matmul_workspace_size(int64_t M, int32_t K, int32_t bits, size_t *bytes);
 int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
                             const uint16_t *biases, int64_t M, int32_t N, int32_t K,
                             int32_t transpose, int32_t group_size, int32_t bits, uint16_t *y,
                             void *workspace, size_t workspace_bytes, void *stream);
+/* the same op with x, scales, biases and y of element type dtype (mi_moe_dtype):
+ * test_quantized_matmul of the reference (fp32, transpose = false) runs through this. */
+int mi_moe_quantized_matmul_typed(const void *x, const uint32_t *w, const void *scales,
+                                  const void *biases, int64_t M, int32_t N, int32_t K,
+                                  int32_t transpose, int32_t group_size, int32_t bits, int32_t dtype,
+                                  void *y, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- R7 silu(gate) * up on bf16 arrays (mlx_sigmoid + mlx_multiply x2,
  * mlx-rs/src/nn/activation.rs:142-144,876-880).  The block itself fuses this into
@@ -227,6 +256,15 @@ int mi_moe_quantize(const float *w, int64_t rows, int64_t cols, int32_t group_si
 int mi_moe_dequantize(const uint32_t *q, const uint16_t *scales, const uint16_t *biases,
                       int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
                       float *w_hat, void *stream);
+/* the same two with scales and biases of element type dtype (mi_moe_dtype): mlx_quantize gives them
+ * the type of its input, float32 in the reference's tests (ops/quantization.rs:298-342).  The codes
+ * come from the fp32 scale and bias either way; the cast to dtype happens afterwards. */
+int mi_moe_quantize_typed(const float *w, int64_t rows, int64_t cols, int32_t group_size,
+                          int32_t bits, int32_t dtype, uint32_t *q, void *scales, void *biases,
+                          void *stream);
+int mi_moe_dequantize_typed(const uint32_t *q, const void *scales, const void *biases, int64_t rows,
+                            int64_t cols, int32_t group_size, int32_t bits, int32_t dtype,
+                            float *w_hat, void *stream);
 
 /* ---- measurement aid; no counterpart in the reference.  A bare streaming kernel with the decode
  * grouped product's access shape (a wave reads a 16 KiB tile from each half of buf, 64 bytes per row

@@ -8,6 +8,7 @@ _SO = os.path.join(_HERE, "libmi_moe.so")
 SCORE_SOFTMAX_THEN_TOPK_RENORM = 0
 SCORE_SOFTMAX_THEN_TOPK = 1
 SCORE_TOPK_THEN_SOFTMAX = 2
+DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 N_STAGES = 6
 N_KERNEL_TIMES = 8
 KERNEL_NAMES = ("gate_up_tiles256", "gate_up_tiles128", "gate_up_tiles64", "gate_up_streamed",
@@ -25,6 +26,7 @@ EXPORTS = (
     "mi_moe_gather_qmm_workspace_size", "mi_moe_gather_qmm",
     "mi_moe_quantized_matmul_workspace_size", "mi_moe_quantized_matmul", "mi_moe_swiglu", "mi_moe_combine",
     "mi_moe_quantize", "mi_moe_dequantize", "mi_moe_stream_probe",
+    "mi_moe_gather_qmm_typed", "mi_moe_quantized_matmul_typed", "mi_moe_quantize_typed", "mi_moe_dequantize_typed",
 )
 
 
@@ -106,6 +108,11 @@ def load_library():
         "mi_moe_quantize": [vp, i64, i64, i32, i32, vp, vp, vp, vp],
         "mi_moe_dequantize": [vp, vp, vp, i64, i64, i32, i32, vp, vp],
         "mi_moe_stream_probe": [vp, sz, vp, vp],
+        "mi_moe_gather_qmm_typed": [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, i32, i32, i32,
+                                    i32, i32, vp, vp, sz, vp],
+        "mi_moe_quantized_matmul_typed": [vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, i32, vp, vp, sz, vp],
+        "mi_moe_quantize_typed": [vp, i64, i64, i32, i32, i32, vp, vp, vp, vp],
+        "mi_moe_dequantize_typed": [vp, vp, vp, i64, i64, i32, i32, i32, vp, vp],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)

@@ -67,18 +67,26 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
+// the block runs on the tuned kernels with 4- or 8-bit codes in groups of 64; other group sizes and
+// 2-bit codes take the plain products
+bool plain_config(const mi_moe_config &c) { return c.group_size != 64 || c.bits == 2; }
+
 int check_config(const mi_moe_config *c) {
   if (!c) return fail("config is NULL");
-  if (c->bits != 4 && c->bits != 8) return fail("bits must be 4 or 8, got %d", c->bits);
-  if (c->group_size != 64) return fail("group_size must be 64, got %d", c->group_size);
+  if (c->bits != 2 && c->bits != 4 && c->bits != 8) return fail("bits must be 2, 4 or 8, got %d", c->bits);
+  if (c->group_size != 32 && c->group_size != 64 && c->group_size != 128)
+    return fail("group_size must be 32, 64 or 128, got %d", c->group_size);
   if (c->hidden <= 0 || c->hidden % 64) return fail("hidden must be a positive multiple of 64, got %d", c->hidden);
   if (c->intermediate <= 0 || c->intermediate % 64)
     return fail("intermediate must be a positive multiple of 64, got %d", c->intermediate);
+  if (c->hidden % c->group_size || c->intermediate % c->group_size)
+    return fail("hidden and intermediate must be multiples of group_size (%d), got %d, %d", c->group_size, c->hidden,
+                c->intermediate);
   if (c->n_experts < 1 || c->n_experts > 512) return fail("n_experts must be in [1, 512], got %d", c->n_experts);
   if (c->top_k < 1 || c->top_k > c->n_experts || c->top_k > 32)
     return fail("top_k must be in [1, min(n_experts, 32)], got %d", c->top_k);
   if (c->score_mode < 0 || c->score_mode > 2) return fail("unknown score_mode %d", c->score_mode);
-  if (c->bits == 4 && (c->hidden % 128 || c->intermediate % 128))
+  if (!plain_config(*c) && c->bits == 4 && (c->hidden % 128 || c->intermediate % 128))
     return fail("4-bit weights need hidden and intermediate to be multiples of 128 (got %d, %d)", c->hidden,
                 c->intermediate);
   return 0;
@@ -117,6 +125,7 @@ struct ForwardWs {
   int tmr;     // segments of at least this many rows are tiled
   void *disp_scratch;
   uint16_t *hh, *y, *xperm, *xnorm;
+  uint16_t *gu;  // plain products only: the gate and the up product, [P, I] each
   size_t bytes;
 };
 
@@ -135,7 +144,7 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   // (the tiled kernel reads scales in 8-byte pieces: rows of scales must be 4-byte aligned, i.e.
   // an even number of groups per row; other shapes stay on the streaming kernel)
   const bool tiled_ok = (c.hidden / 64) % 2 == 0 && (c.intermediate / 64) % 2 == 0;
-  f.tiled = tiled_ok && tiled_batch(P, c.n_experts, c.bits);
+  f.tiled = tiled_ok && !plain_config(c) && tiled_batch(P, c.n_experts, c.bits);
   f.heavy = f.tiled && heavy_batch(P, c.n_experts, c.bits);
   const int tmr = f.tmr = tile_min_rows(c.bits, f.heavy);
   f.max_mtiles = f.tiled ? (int)(P / kBigTileM + (P / tmr < c.n_experts ? P / tmr : c.n_experts)) : 0;
@@ -148,6 +157,7 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.y = cv.take<uint16_t>((size_t)P * c.hidden);
   f.xperm = cv.take<uint16_t>(f.tiled && c.bits == 4 ? (size_t)T * c.hidden : 0);
   f.xnorm = cv.take<uint16_t>((size_t)T * c.hidden);  // rms_norm(x) of the residual variant
+  f.gu = cv.take<uint16_t>(plain_config(c) ? 2 * (size_t)P * c.intermediate : 0);
   f.bytes = cv.off;
   return f;
 }
@@ -349,7 +359,20 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   d.y = f.y;
   d.N = c.hidden;
   d.K = c.intermediate;
-  if (large_qmm_applies(a) && !ev) {
+  if (plain_config(c)) {
+    // group sizes 32 / 128 or 2-bit codes: the plain products, one output row per sorted pair.  Row r of
+    // the sorted order belongs to pair perm[r], token src_of[r], expert topk_idx[perm[r]].
+    const size_t PI = (size_t)P * c.intermediate;
+    MI_HIP(launch_qmm_plain(x, h->w.gate.w, h->w.gate.scales, h->w.gate.biases, f.src_of, f.topk_idx, f.perm, nullptr,
+                            P, 1, c.intermediate, c.hidden, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.gu, st));
+    MI_HIP(launch_qmm_plain(x, h->w.up.w, h->w.up.scales, h->w.up.biases, f.src_of, f.topk_idx, f.perm, nullptr, P, 1,
+                            c.intermediate, c.hidden, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.gu + PI, st));
+    MI_HIP(launch_swiglu(f.gu, f.gu + PI, (int64_t)PI, f.hh, st));
+    MI_STAGE_DONE();
+    MI_HIP(launch_qmm_plain(f.hh, h->w.down.w, h->w.down.scales, h->w.down.biases, nullptr, f.topk_idx, f.perm, f.perm,
+                            P, 1, c.hidden, c.intermediate, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.y, st));
+    MI_STAGE_DONE();
+  } else if (large_qmm_applies(a) && !ev) {
     // Four chains that share no rows: the three tile classes and the streamed segments, each
     // gate/up then down.  The short classes leave most of the chip idle when they run alone
     // (a few dozen workgroups of 64 K steps each); side by side they fill it.  The chain that is
@@ -608,37 +631,45 @@ int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M
   return 0;
 } MI_CATCH("gather_qmm_workspace_size")
 
-int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
-                      const uint16_t *biases, const uint32_t *lhs_indices, const uint32_t *rhs_indices,
-                      int64_t n_idx, int64_t x_batch, int32_t M, int32_t N, int32_t K, int32_t n_experts,
-                      int32_t transpose, int32_t group_size, int32_t bits, int32_t sorted_indices,
-                      uint16_t *y, void *workspace, size_t workspace_bytes, void *stream) try {
-  (void)sorted_indices;  // a hint in MLX; the segments are rebuilt here either way
-  (void)x_batch;
-  if (bits != 4 && bits != 8) return fail("gather_qmm: bits must be 4 or 8, got %d", bits);
-  if (group_size != 64) return fail("gather_qmm: group_size must be 64, got %d", group_size);
-  if (!transpose) {  // w [E, K, N*bits/32]: the plain kernel, no workspace
-    if (K <= 0) return fail("gather_qmm: K must be positive, got %d", K);
-    if (N <= 0 || N % 64) return fail("gather_qmm: with transpose = false N must be a positive multiple of 64, got %d", N);
-    if (M < 1) return fail("gather_qmm: M must be positive, got %d", M);
-    if (n_experts < 1) return fail("gather_qmm: n_experts must be positive, got %d", n_experts);
-    if (n_idx < 0 || n_idx * M > (int64_t)1 << 30) return fail("gather_qmm: index count out of range");
-    if (n_idx == 0) return 0;
-    if (!x || !w || !scales || !biases || !y) return fail("gather_qmm: x, w, scales, biases and y must be non-NULL");
-    if (!rhs_indices) return fail("gather_qmm: rhs_indices is required");
-    MI_HIP(launch_qmm_nt(x, w, scales, biases, lhs_indices, rhs_indices, n_idx * M, M, N, K, group_size, bits, y,
-                         static_cast<hipStream_t>(stream)));
-    return 0;
-  }
-  if (K <= 0 || K % 64) return fail("gather_qmm: K must be a positive multiple of 64, got %d", K);
-  if (bits == 4 && K % 128) return fail("gather_qmm: 4-bit weights need K to be a multiple of 128, got %d", K);
-  if (N <= 0 || N % 16) return fail("gather_qmm: N must be a positive multiple of 16, got %d", N);
+// which products the tuned kernels take; everything else goes to the plain ones
+static bool tuned_shape(int32_t dtype, int32_t transpose, int32_t group_size, int32_t bits, int32_t N, int32_t K) {
+  return dtype == MI_MOE_DTYPE_BF16 && transpose && group_size == 64 && (bits == 4 || bits == 8) && K % 64 == 0 &&
+         (bits != 4 || K % 128 == 0) && N % 16 == 0;
+}
+
+static int check_qmm_shape(const char *who, int32_t dtype, int32_t transpose, int32_t group_size, int32_t bits,
+                           int32_t N, int32_t K) {
+  if (dtype != MI_MOE_DTYPE_BF16 && dtype != MI_MOE_DTYPE_F16 && dtype != MI_MOE_DTYPE_F32)
+    return fail("%s: dtype must be MI_MOE_DTYPE_BF16, _F16 or _F32, got %d", who, dtype);
+  if (bits != 2 && bits != 4 && bits != 8) return fail("%s: bits must be 2, 4 or 8, got %d", who, bits);
+  if (group_size != 32 && group_size != 64 && group_size != 128)
+    return fail("%s: group_size must be 32, 64 or 128, got %d", who, group_size);
+  if (K <= 0 || N <= 0) return fail("%s: N and K must be positive, got %d, %d", who, N, K);
+  // the quantised axis: K with transpose = true (w [N, K*bits/32]), N otherwise (w [K, N*bits/32])
+  const int32_t q_axis = transpose ? K : N;
+  if (q_axis % group_size)
+    return fail("%s: %s (%d) must be a multiple of group_size (%d)", who, transpose ? "K" : "N", q_axis, group_size);
+  return 0;
+}
+
+static int gather_qmm_impl(const void *x, const uint32_t *w, const void *scales, const void *biases,
+                           const uint32_t *lhs_indices, const uint32_t *rhs_indices, int64_t n_idx, int32_t M,
+                           int32_t N, int32_t K, int32_t n_experts, int32_t transpose, int32_t group_size,
+                           int32_t bits, int32_t dtype, void *y, void *workspace, size_t workspace_bytes,
+                           void *stream) {
+  if (check_qmm_shape("gather_qmm", dtype, transpose, group_size, bits, N, K)) return 1;
   if (M < 1) return fail("gather_qmm: M must be positive, got %d", M);
-  if (n_experts < 1 || n_experts > 512) return fail("gather_qmm: n_experts must be in [1, 512], got %d", n_experts);
+  if (n_experts < 1) return fail("gather_qmm: n_experts must be positive, got %d", n_experts);
   if (n_idx < 0 || n_idx * M > (int64_t)1 << 30) return fail("gather_qmm: index count out of range");
   if (n_idx == 0) return 0;
   if (!x || !w || !scales || !biases || !y) return fail("gather_qmm: x, w, scales, biases and y must be non-NULL");
   if (!rhs_indices) return fail("gather_qmm: rhs_indices is required");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!tuned_shape(dtype, transpose, group_size, bits, N, K) || n_experts > 512) {  // the plain kernels, no workspace
+    MI_HIP(launch_qmm_plain(x, w, scales, biases, lhs_indices, rhs_indices, nullptr, nullptr, n_idx * M, M, N, K,
+                            group_size, bits, transpose != 0, dtype, y, st));
+    return 0;
+  }
   if (!aligned16(x) || !aligned16(w) || !aligned16(scales) || !aligned16(biases) || !aligned16(y))
     return fail("gather_qmm: pointers must be 16-byte aligned");
   const int64_t rows = n_idx * M;
@@ -653,18 +684,17 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   uint32_t *perm = cv.take<uint32_t>((size_t)rows);
   uint32_t *src_rows = cv.take<uint32_t>((size_t)rows);
   uint32_t *dst_rows = cv.take<uint32_t>((size_t)rows);
-  hipStream_t st = static_cast<hipStream_t>(stream);
   MI_HIP(launch_dispatch(rhs_indices, n_idx, n_experts, 1, counts, offsets, perm, nullptr, nullptr, work,
                          nullptr, 0, 0, scratch, st));
   MI_HIP(launch_row_maps(perm, lhs_indices, offsets, n_idx, M, n_experts, src_rows, dst_rows, work, st));
   GroupedArgs a{};
-  a.x = x;
+  a.x = static_cast<const uint16_t *>(x);
   a.src_rows = src_rows;
   a.dst_rows = dst_rows;
   a.work = work;
   a.max_active = (int)(n_idx < n_experts ? n_idx : n_experts);
-  a.w0 = w; a.s0 = scales; a.b0 = biases;
-  a.y = y;
+  a.w0 = w; a.s0 = static_cast<const uint16_t *>(scales); a.b0 = static_cast<const uint16_t *>(biases);
+  a.y = static_cast<uint16_t *>(y);
   a.N = N;
   a.K = K;
   a.bits = bits;
@@ -672,7 +702,29 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
   a.max_rows_per_expert = rows;
   MI_HIP(launch_grouped_qmm(a, false, st));
   return 0;
+}
+
+int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                      const uint16_t *biases, const uint32_t *lhs_indices, const uint32_t *rhs_indices,
+                      int64_t n_idx, int64_t x_batch, int32_t M, int32_t N, int32_t K, int32_t n_experts,
+                      int32_t transpose, int32_t group_size, int32_t bits, int32_t sorted_indices,
+                      uint16_t *y, void *workspace, size_t workspace_bytes, void *stream) try {
+  (void)sorted_indices;  // a hint in MLX; the segments are rebuilt here either way
+  (void)x_batch;
+  return gather_qmm_impl(x, w, scales, biases, lhs_indices, rhs_indices, n_idx, M, N, K, n_experts, transpose,
+                         group_size, bits, MI_MOE_DTYPE_BF16, y, workspace, workspace_bytes, stream);
 } MI_CATCH("gather_qmm")
+
+int mi_moe_gather_qmm_typed(const void *x, const uint32_t *w, const void *scales, const void *biases,
+                            const uint32_t *lhs_indices, const uint32_t *rhs_indices, int64_t n_idx,
+                            int64_t x_batch, int32_t M, int32_t N, int32_t K, int32_t n_experts,
+                            int32_t transpose, int32_t group_size, int32_t bits, int32_t sorted_indices,
+                            int32_t dtype, void *y, void *workspace, size_t workspace_bytes, void *stream) try {
+  (void)sorted_indices;
+  (void)x_batch;
+  return gather_qmm_impl(x, w, scales, biases, lhs_indices, rhs_indices, n_idx, M, N, K, n_experts, transpose,
+                         group_size, bits, dtype, y, workspace, workspace_bytes, stream);
+} MI_CATCH("gather_qmm_typed")
 
 static size_t qmm_dense_bytes(int64_t M, int32_t K, int32_t bits, size_t *mt_words) {
   const size_t ntiles = (size_t)((M + kBigTileM - 1) / kBigTileM);
@@ -690,28 +742,20 @@ int mi_moe_quantized_matmul_workspace_size(int64_t M, int32_t K, int32_t bits, s
   return 0;
 } MI_CATCH("quantized_matmul_workspace_size")
 
-int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
-                            const uint16_t *biases, int64_t M, int32_t N, int32_t K, int32_t transpose,
-                            int32_t group_size, int32_t bits, uint16_t *y, void *workspace,
-                            size_t workspace_bytes, void *stream) try {
-  if (bits != 4 && bits != 8) return fail("quantized_matmul: bits must be 4 or 8, got %d", bits);
-  if (group_size != 64) return fail("quantized_matmul: group_size must be 64, got %d", group_size);
-  if (!transpose) {  // w [K, N*bits/32]: the plain kernel, no workspace
-    if (K <= 0) return fail("quantized_matmul: K must be positive, got %d", K);
-    if (N <= 0 || N % 64) return fail("quantized_matmul: with transpose = false N must be a positive multiple of 64, got %d", N);
-    if (M < 0 || M > (int64_t)1 << 30) return fail("quantized_matmul: row count out of range");
-    if (M == 0) return 0;
-    if (!x || !w || !scales || !biases || !y) return fail("quantized_matmul: x, w, scales, biases and y must be non-NULL");
-    MI_HIP(launch_qmm_nt(x, w, scales, biases, nullptr, nullptr, M, 1, N, K, group_size, bits, y,
-                         static_cast<hipStream_t>(stream)));
-    return 0;
-  }
-  if (K <= 0 || K % 64) return fail("quantized_matmul: K must be a positive multiple of 64, got %d", K);
-  if (bits == 4 && K % 128) return fail("quantized_matmul: 4-bit weights need K to be a multiple of 128, got %d", K);
-  if (N <= 0 || N % 16) return fail("quantized_matmul: N must be a positive multiple of 16, got %d", N);
+static int quantized_matmul_impl(const void *x, const uint32_t *w, const void *scales, const void *biases,
+                                 int64_t M, int32_t N, int32_t K, int32_t transpose, int32_t group_size,
+                                 int32_t bits, int32_t dtype, void *y, void *workspace, size_t workspace_bytes,
+                                 void *stream) {
+  if (check_qmm_shape("quantized_matmul", dtype, transpose, group_size, bits, N, K)) return 1;
   if (M < 0 || M > (int64_t)1 << 30) return fail("quantized_matmul: row count out of range");
   if (M == 0) return 0;
   if (!x || !w || !scales || !biases || !y) return fail("quantized_matmul: x, w, scales, biases and y must be non-NULL");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!tuned_shape(dtype, transpose, group_size, bits, N, K)) {  // the plain kernels, no workspace
+    MI_HIP(launch_qmm_plain(x, w, scales, biases, nullptr, nullptr, nullptr, nullptr, M, 1, N, K, group_size, bits,
+                            transpose != 0, dtype, y, st));
+    return 0;
+  }
   if (!aligned16(x) || !aligned16(w) || !aligned16(scales) || !aligned16(biases) || !aligned16(y))
     return fail("quantized_matmul: pointers must be 16-byte aligned");
   size_t mt_words = 0;
@@ -722,21 +766,21 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
   uint32_t *mtiles = cv.take<uint32_t>(mt_words);
   // one segment of M rows: the tiled kernel from the batch threshold on (fewer rows: streaming passes)
   const bool big = M >= tiled_avg_rows(bits) && (K / 64) % 2 == 0;
+  const uint16_t *xb = static_cast<const uint16_t *>(x);
   uint16_t *xperm = (bits == 4 && big) ? cv.take<uint16_t>((size_t)M * K) : nullptr;
-  hipStream_t st = static_cast<hipStream_t>(stream);
   const int cap256 = (int)((M + kBigTileM - 1) / kBigTileM);
   MI_HIP(launch_dense_records(M, big ? tiled_avg_rows(bits) : 0, work, mtiles, cap256, st));
-  if (xperm) MI_HIP(launch_pair_rows(x, M, K, xperm, st));
+  if (xperm) MI_HIP(launch_pair_rows(xb, M, K, xperm, st));
   GroupedArgs a{};
-  a.x = x;
-  a.x_perm = bits == 4 ? xperm : x;
+  a.x = xb;
+  a.x_perm = bits == 4 ? xperm : xb;
   a.work = work;
   a.max_active = 1;
   a.mtiles = big ? mtiles : nullptr;
   a.max_mtiles = big ? cap256 : 0;
   a.tile_cap_e = big ? 1 : 0;
-  a.w0 = w; a.s0 = scales; a.b0 = biases;
-  a.y = y;
+  a.w0 = w; a.s0 = static_cast<const uint16_t *>(scales); a.b0 = static_cast<const uint16_t *>(biases);
+  a.y = static_cast<uint16_t *>(y);
   a.N = N;
   a.K = K;
   a.bits = bits;
@@ -744,7 +788,23 @@ int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t
   a.max_rows_per_expert = M;
   MI_HIP(launch_grouped_qmm(a, false, st));
   return 0;
+}
+
+int mi_moe_quantized_matmul(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
+                            const uint16_t *biases, int64_t M, int32_t N, int32_t K, int32_t transpose,
+                            int32_t group_size, int32_t bits, uint16_t *y, void *workspace,
+                            size_t workspace_bytes, void *stream) try {
+  return quantized_matmul_impl(x, w, scales, biases, M, N, K, transpose, group_size, bits, MI_MOE_DTYPE_BF16, y,
+                               workspace, workspace_bytes, stream);
 } MI_CATCH("quantized_matmul")
+
+int mi_moe_quantized_matmul_typed(const void *x, const uint32_t *w, const void *scales, const void *biases,
+                                  int64_t M, int32_t N, int32_t K, int32_t transpose, int32_t group_size,
+                                  int32_t bits, int32_t dtype, void *y, void *workspace, size_t workspace_bytes,
+                                  void *stream) try {
+  return quantized_matmul_impl(x, w, scales, biases, M, N, K, transpose, group_size, bits, dtype, y, workspace,
+                               workspace_bytes, stream);
+} MI_CATCH("quantized_matmul_typed")
 
 int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out, void *stream) try {
   if (n < 0) return fail("swiglu: negative element count");
@@ -785,22 +845,39 @@ static int check_quant_args(const char *who, int64_t rows, int64_t cols, int32_t
   return 0;
 }
 
-int mi_moe_quantize(const float *w, int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
-                    uint32_t *q, uint16_t *scales, uint16_t *biases, void *stream) try {
-  if (check_quant_args("quantize", rows, cols, group_size, bits)) return 1;
+static int check_dtype(const char *who, int32_t dtype) {
+  if (dtype != MI_MOE_DTYPE_BF16 && dtype != MI_MOE_DTYPE_F16 && dtype != MI_MOE_DTYPE_F32)
+    return fail("%s: dtype must be MI_MOE_DTYPE_BF16, _F16 or _F32, got %d", who, dtype);
+  return 0;
+}
+
+int mi_moe_quantize_typed(const float *w, int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
+                          int32_t dtype, uint32_t *q, void *scales, void *biases, void *stream) try {
+  if (check_quant_args("quantize", rows, cols, group_size, bits) || check_dtype("quantize", dtype)) return 1;
   if (rows * cols == 0) return 0;
   if (!w || !q || !scales || !biases) return fail("quantize: w, q, scales and biases must be non-NULL");
-  MI_HIP(launch_quantize(w, rows, cols, group_size, bits, q, scales, biases, static_cast<hipStream_t>(stream)));
+  MI_HIP(launch_quantize(w, rows, cols, group_size, bits, q, scales, biases, dtype, static_cast<hipStream_t>(stream)));
   return 0;
+} MI_CATCH("quantize_typed")
+
+int mi_moe_quantize(const float *w, int64_t rows, int64_t cols, int32_t group_size, int32_t bits,
+                    uint32_t *q, uint16_t *scales, uint16_t *biases, void *stream) try {
+  return mi_moe_quantize_typed(w, rows, cols, group_size, bits, MI_MOE_DTYPE_BF16, q, scales, biases, stream);
 } MI_CATCH("quantize")
+
+int mi_moe_dequantize_typed(const uint32_t *q, const void *scales, const void *biases, int64_t rows,
+                            int64_t cols, int32_t group_size, int32_t bits, int32_t dtype, float *w_hat,
+                            void *stream) try {
+  if (check_quant_args("dequantize", rows, cols, group_size, bits) || check_dtype("dequantize", dtype)) return 1;
+  if (rows * cols == 0) return 0;
+  if (!q || !scales || !biases || !w_hat) return fail("dequantize: q, scales, biases and w_hat must be non-NULL");
+  MI_HIP(launch_dequantize(q, scales, biases, rows, cols, group_size, bits, w_hat, dtype, static_cast<hipStream_t>(stream)));
+  return 0;
+} MI_CATCH("dequantize_typed")
 
 int mi_moe_dequantize(const uint32_t *q, const uint16_t *scales, const uint16_t *biases, int64_t rows,
                       int64_t cols, int32_t group_size, int32_t bits, float *w_hat, void *stream) try {
-  if (check_quant_args("dequantize", rows, cols, group_size, bits)) return 1;
-  if (rows * cols == 0) return 0;
-  if (!q || !scales || !biases || !w_hat) return fail("dequantize: q, scales, biases and w_hat must be non-NULL");
-  MI_HIP(launch_dequantize(q, scales, biases, rows, cols, group_size, bits, w_hat, static_cast<hipStream_t>(stream)));
-  return 0;
+  return mi_moe_dequantize_typed(q, scales, biases, rows, cols, group_size, bits, MI_MOE_DTYPE_BF16, w_hat, stream);
 } MI_CATCH("dequantize")
 
 }  // extern "C"

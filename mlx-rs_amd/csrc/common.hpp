@@ -263,13 +263,17 @@ hipError_t launch_combine(const uint16_t *y, const uint16_t *scores, const uint3
                           hipStream_t st);
 hipError_t launch_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_t T, int H,
                            uint16_t *out, hipStream_t st);
-hipError_t launch_qmm_nt(const uint16_t *x, const uint32_t *w, const uint16_t *scales,
-                         const uint16_t *biases, const uint32_t *lhs, const uint32_t *rhs, int64_t rows,
-                         int M, int N, int K, int group, int bits, uint16_t *y, hipStream_t st);
+// plain products (any float type, group sizes 32 / 64 / 128, 2 / 4 / 8 bits, both weight layouts);
+// dt: 0 bf16, 1 fp16, 2 fp32.  Output row r = j * M + m: expert rhs[rhs_map ? rhs_map[j] : j] (0 without
+// rhs), x row (lhs ? lhs[j] : j) * M + m, destination row dst_map ? dst_map[r] : r.
+hipError_t launch_qmm_plain(const void *x, const uint32_t *w, const void *scales, const void *biases,
+                            const uint32_t *lhs, const uint32_t *rhs, const uint32_t *rhs_map,
+                            const uint32_t *dst_map, int64_t rows, int M, int N, int K, int group, int bits,
+                            bool transpose, int dt, void *y, hipStream_t st);
 hipError_t launch_quantize(const float *w, int64_t rows, int64_t cols, int group, int bits,
-                           uint32_t *q, uint16_t *s, uint16_t *b, hipStream_t st);
-hipError_t launch_dequantize(const uint32_t *q, const uint16_t *s, const uint16_t *b,
-                             int64_t rows, int64_t cols, int group, int bits, float *out,
+                           uint32_t *q, void *s, void *b, int dt, hipStream_t st);
+hipError_t launch_dequantize(const uint32_t *q, const void *s, const void *b,
+                             int64_t rows, int64_t cols, int group, int bits, float *out, int dt,
                              hipStream_t st);
 
 }  // namespace mi_moe

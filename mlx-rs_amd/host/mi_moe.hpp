@@ -25,6 +25,7 @@
 #include <stdexcept>
 #include <string>
 #include <tuple>
+#include <algorithm>
 #include <utility>
 #include <variant>
 #include <vector>
@@ -69,8 +70,8 @@ inline Exception hip_error(const char *who, hipError_t e) {
 }
 }  // namespace detail
 
-enum class Dtype { Bfloat16, Float32, Uint32 };
-inline size_t size_of(Dtype d) { return d == Dtype::Bfloat16 ? 2 : 4; }
+enum class Dtype { Bfloat16, Float16, Float32, Uint32 };
+inline size_t size_of(Dtype d) { return d == Dtype::Bfloat16 || d == Dtype::Float16 ? 2 : 4; }
 
 struct Stream {
   hipStream_t handle = nullptr;  // nullptr = the default stream
@@ -238,9 +239,77 @@ inline Result<Array> quantized_matmul(const Array &x, const Array &w, const Arra
   return y;
 }
 
+// the library's code of a floating element type, or -1
+inline int32_t float_code(Dtype d) {
+  return d == Dtype::Bfloat16 ? MI_MOE_DTYPE_BF16 : d == Dtype::Float16 ? MI_MOE_DTYPE_F16
+       : d == Dtype::Float32 ? MI_MOE_DTYPE_F32 : -1;
+}
+
+namespace idx {
+// index array `a` (or, when absent, 0, 1, ... in the shape `counted`) on the host, with its shape
+inline Result<std::pair<std::vector<uint32_t>, std::vector<int64_t>>> host_indices(const Array *a,
+                                                                                  const std::vector<int64_t> &counted,
+                                                                                  Stream s) {
+  std::pair<std::vector<uint32_t>, std::vector<int64_t>> r;
+  if (a) {
+    if (a->dtype() != Dtype::Uint32) return Exception("gather_qmm: index arrays must be uint32");
+    r.first.resize((size_t)a->size());
+    r.second = a->shape();
+    if (a->size()) {
+      auto c = a->to_host(r.first.data(), s);
+      if (c.is_err()) return c.error();
+    }
+  } else {
+    int64_t n = 1;
+    for (int64_t d : counted) n *= d;
+    r.first.resize((size_t)n);
+    std::iota(r.first.begin(), r.first.end(), 0u);
+    r.second = counted;
+  }
+  return r;
+}
+// numpy-style broadcast of two shapes (aligned at the last axis); empty optional: they do not broadcast
+inline std::optional<std::vector<int64_t>> broadcast_shape(const std::vector<int64_t> &a, const std::vector<int64_t> &b) {
+  const size_t n = std::max(a.size(), b.size());
+  std::vector<int64_t> out(n);
+  for (size_t i = 0; i < n; ++i) {
+    const int64_t da = i < n - a.size() ? 1 : a[i - (n - a.size())];
+    const int64_t db = i < n - b.size() ? 1 : b[i - (n - b.size())];
+    if (da != db && da != 1 && db != 1) return std::nullopt;
+    out[i] = da == 1 ? db : da;
+  }
+  return out;
+}
+// the elements of `v` (shape `from`) as an array of shape `to` (a broadcast of `from`), flattened
+inline std::vector<uint32_t> broadcast_to(const std::vector<uint32_t> &v, const std::vector<int64_t> &from,
+                                          const std::vector<int64_t> &to) {
+  int64_t n = 1;
+  for (int64_t d : to) n *= d;
+  std::vector<uint32_t> out((size_t)n);
+  const size_t off = to.size() - from.size();
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t rem = i, src = 0, stride = 1;
+    for (size_t ax = to.size(); ax-- > 0;) {
+      const int64_t c = rem % to[ax];
+      rem /= to[ax];
+      if (ax >= off) {
+        const int64_t d = from[ax - off];
+        src += (d == 1 ? 0 : c) * stride;
+        stride *= d;
+      }
+    }
+    out[(size_t)i] = v[(size_t)src];
+  }
+  return out;
+}
+}  // namespace idx
+
 // gather_qmm(x, w, scales, biases, lhs_indices, rhs_indices, transpose, group_size, bits,
-// sorted_indices): x bf16 [x_batch, M, K]; w u32 [E, N, K*bits/32]; indices u32 [n_idx];
-// returns bf16 [n_idx, M, N].
+// sorted_indices) with the batch semantics of mlx-rs/src/ops/quantization.rs:160-230: x is
+// [..., M, K] in bf16, f16 or f32 (scales and biases in the same type), w u32 [..., N, K*bits/32]
+// (transpose = false: [..., K, N*bits/32]); the leading axes are batch axes which the uint32 index
+// arrays (any shapes, broadcast against each other; an absent one counts through its batch) index in
+// flattened form.  Returns [*broadcast shape, M, N].  The index arrays pass through the host.
 inline Result<Array> gather_qmm(const Array &x, const Array &w, const Array &scales,
                                 const Array *biases = nullptr, const Array *lhs_indices = nullptr,
                                 const Array *rhs_indices = nullptr,
@@ -250,29 +319,49 @@ inline Result<Array> gather_qmm(const Array &x, const Array &w, const Array &sca
                                 std::optional<bool> sorted_indices = {}, Stream s = {}) {
   const bool tr = transpose.value_or(true), sorted = sorted_indices.value_or(false);
   const int32_t g = group_size.value_or(DEFAULT_GROUP_SIZE), b = bits.value_or(DEFAULT_BITS);
-  if (auto e = detail::want(x, Dtype::Bfloat16, "gather_qmm", "x")) return *e;
+  const int32_t dt = float_code(x.dtype());
+  if (dt < 0) return Exception("gather_qmm: x has the wrong dtype (bfloat16, float16 or float32)");
   if (auto e = detail::want(w, Dtype::Uint32, "gather_qmm", "w")) return *e;
-  if (auto e = detail::want(scales, Dtype::Bfloat16, "gather_qmm", "scales")) return *e;
+  if (auto e = detail::want(scales, x.dtype(), "gather_qmm", "scales")) return *e;
   if (!biases) return Exception("gather_qmm: biases are required in affine mode");
-  if (!rhs_indices) return Exception("gather_qmm: rhs_indices is required");
-  if (x.ndim() != 3 || w.ndim() != 3)
-    return Exception("gather_qmm: x must be [batch, M, K] and w [E, N, K*bits/32]");
-  const int64_t n_idx = rhs_indices->size(), xb = x.dim(0);
-  const int32_t M = (int32_t)x.dim(1), K = (int32_t)x.dim(2);
-  const int32_t E = (int32_t)w.dim(0), N = tr ? (int32_t)w.dim(1) : (int32_t)(w.dim(2) * 32 / b);
+  if (auto e = detail::want(*biases, x.dtype(), "gather_qmm", "biases")) return *e;
+  if (x.ndim() < 2 || w.ndim() < 2 || b <= 0)
+    return Exception("gather_qmm: x must be [..., M, K] and w [..., N, K*bits/32]");
+  const std::vector<int64_t> xb_shape(x.shape().begin(), x.shape().end() - 2), wb_shape(w.shape().begin(), w.shape().end() - 2);
+  int64_t xb = 1, E = 1;
+  for (int64_t d : xb_shape) xb *= d;
+  for (int64_t d : wb_shape) E *= d;
+  const int32_t M = (int32_t)x.dim(-2), K = (int32_t)x.dim(-1);
+  const int32_t N = tr ? (int32_t)w.dim(-2) : (int32_t)(w.dim(-1) * 32 / b);
+  auto lh = idx::host_indices(lhs_indices, xb_shape, s);
+  if (lh.is_err()) return lh.error();
+  auto rh = idx::host_indices(rhs_indices, wb_shape, s);
+  if (rh.is_err()) return rh.error();
+  const auto bshape = idx::broadcast_shape(lh.value().second, rh.value().second);
+  if (!bshape) return Exception("gather_qmm: the shapes of lhs_indices and rhs_indices do not broadcast");
+  const std::vector<uint32_t> lf = idx::broadcast_to(lh.value().first, lh.value().second, *bshape);
+  const std::vector<uint32_t> rf = idx::broadcast_to(rh.value().first, rh.value().second, *bshape);
+  const int64_t n_idx = (int64_t)rf.size();
+  std::vector<int64_t> out_shape = *bshape;
+  out_shape.push_back(M);
+  out_shape.push_back(N);
+  auto y = Array::empty(out_shape, x.dtype());
+  if (y.is_err() || n_idx == 0) return y;
+  auto ld = Array::from_host(lf.data(), {n_idx}, Dtype::Uint32, s);
+  auto rd = Array::from_host(rf.data(), {n_idx}, Dtype::Uint32, s);
+  if (ld.is_err()) return ld;
+  if (rd.is_err()) return rd;
   size_t ws_bytes = 0;
-  if (mi_moe_gather_qmm_workspace_size(E, n_idx, M, &ws_bytes)) return detail::last_error("gather_qmm");
-  auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);
-  auto y = Array::empty({n_idx, (int64_t)M, (int64_t)N}, Dtype::Bfloat16);
-  if (ws.is_err()) return ws;
-  if (y.is_err()) return y;
-  if (mi_moe_gather_qmm(x.ptr<uint16_t>(), w.ptr<uint32_t>(), scales.ptr<uint16_t>(),
-                        biases->ptr<uint16_t>(), lhs_indices ? lhs_indices->ptr<uint32_t>() : nullptr,
-                        rhs_indices->ptr<uint32_t>(), n_idx, xb, M, N, K, E, tr ? 1 : 0, g, b,
-                        sorted ? 1 : 0, y.value().ptr<uint16_t>(), ws.value().data(),
-                        ws.value().nbytes(), s.as_ptr()))
+  if (mi_moe_gather_qmm_workspace_size((int32_t)std::min<int64_t>(std::max<int64_t>(E, 1), 512), n_idx, M, &ws_bytes))
     return detail::last_error("gather_qmm");
-  // the workspace may be released only after the work that uses it has finished
+  auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);
+  if (ws.is_err()) return ws;
+  if (mi_moe_gather_qmm_typed(x.data(), w.ptr<uint32_t>(), scales.data(), biases->data(), ld.value().ptr<uint32_t>(),
+                              rd.value().ptr<uint32_t>(), n_idx, xb, M, N, K, (int32_t)E, tr ? 1 : 0, g, b,
+                              sorted ? 1 : 0, dt, y.value().data(), ws.value().data(), ws.value().nbytes(),
+                              s.as_ptr()))
+    return detail::last_error("gather_qmm");
+  // the workspace and the index copies may be released only after the work that uses them has finished
   if (hipError_t e = hipStreamSynchronize(s.handle); e != hipSuccess)
     return detail::hip_error("gather_qmm", e);
   return y;

@@ -2,8 +2,9 @@
 dispatch each one replaces.  torch supplies device memory and the current stream; all
 arithmetic happens in libmi_moe.so.
 
-dtypes: activations/scales/biases ``torch.bfloat16``; packed weights and indices
-``torch.int32`` holding the uint32 bit patterns (torch has no arithmetic on uint32).
+dtypes: activations/scales/biases ``torch.bfloat16`` on the hot path (the op-level functions also
+take float16 and float32); packed weights and indices ``torch.int32`` holding the uint32 bit
+patterns (torch has no arithmetic on uint32).
 """
 import ctypes as C
 
@@ -35,83 +36,134 @@ def _workspace(nbytes, device):
     return torch.empty(int(nbytes) + 256, dtype=torch.uint8, device=device)
 
 
-def quantize(w, group_size=64, bits=4):
-    """ops::quantize (mlx-rs/src/ops/quantization.rs:50-83): returns (w_q, scales, biases)."""
+_DTYPES = {torch.bfloat16: capi.DTYPE_BF16, torch.float16: capi.DTYPE_F16, torch.float32: capi.DTYPE_F32}
+
+
+def _float_dtype(t, name):
+    if t.dtype not in _DTYPES:
+        raise capi.MoeError(f"{name}: expected bfloat16, float16 or float32, got {t.dtype}")
+    if not t.is_cuda:
+        raise capi.MoeError(f"{name}: expected a device tensor")
+    if not t.is_contiguous():
+        raise capi.MoeError(f"{name}: expected a contiguous tensor")
+    return _DTYPES[t.dtype]
+
+
+def quantize(w, group_size=64, bits=4, dtype=torch.bfloat16):
+    """ops::quantize (mlx-rs/src/ops/quantization.rs:50-83): returns (w_q, scales, biases).
+    w: float32 [rows, cols]; scales and biases come out in ``dtype`` (MLX gives them the type of its
+    input: pass torch.float32 for the reference's float32 flows)."""
     lib = load_library()
     _need(w, torch.float32, "w")
+    if dtype not in _DTYPES:
+        raise capi.MoeError(f"quantize: dtype must be bfloat16, float16 or float32, got {dtype}")
     rows, cols = w.shape
     if cols % max(group_size, 1) or group_size not in (32, 64, 128) or bits not in (2, 4, 8):
         check(lib.mi_moe_quantize(None, rows, cols, group_size, bits, None, None, None, None))
     q = torch.empty((rows, cols * bits // 32), dtype=torch.int32, device=w.device)
-    s = torch.empty((rows, cols // group_size), dtype=torch.bfloat16, device=w.device)
+    s = torch.empty((rows, cols // group_size), dtype=dtype, device=w.device)
     b = torch.empty_like(s)
-    check(lib.mi_moe_quantize(_ptr(w), rows, cols, group_size, bits, _ptr(q), _ptr(s), _ptr(b), _stream()))
+    check(lib.mi_moe_quantize_typed(_ptr(w), rows, cols, group_size, bits, _DTYPES[dtype], _ptr(q), _ptr(s), _ptr(b),
+                                    _stream()))
     return q, s, b
 
 
 def dequantize(w_q, scales, biases, group_size=64, bits=4):
-    """ops::dequantize (mlx-rs/src/ops/quantization.rs:124-158), fp32 result."""
+    """ops::dequantize (mlx-rs/src/ops/quantization.rs:124-158), fp32 result; scales and biases in
+    bfloat16, float16 or float32."""
     lib = load_library()
     _need(w_q, torch.int32, "w_q")
+    dt = _float_dtype(scales, "scales")
+    _need(biases, scales.dtype, "biases")
     rows = w_q.shape[0]
     cols = w_q.shape[1] * 32 // bits
     out = torch.empty((rows, cols), dtype=torch.float32, device=w_q.device)
-    check(lib.mi_moe_dequantize(_ptr(w_q), _ptr(_need(scales, torch.bfloat16, "scales")),
-                                _ptr(_need(biases, torch.bfloat16, "biases")), rows, cols, group_size,
-                                bits, _ptr(out), _stream()))
+    check(lib.mi_moe_dequantize_typed(_ptr(w_q), _ptr(scales), _ptr(biases), rows, cols, group_size, bits, dt,
+                                      _ptr(out), _stream()))
     return out
+
+
+def _prod(shape):
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return n
 
 
 def gather_qmm(x, w, scales, biases, lhs_indices=None, rhs_indices=None, transpose=True,
                group_size=64, bits=4, sorted_indices=False):
-    """ops::gather_qmm (mlx-rs/src/ops/quantization.rs:160-230), same argument order and
-    defaults.  x: bf16 [x_batch, M, K]; w: int32 [E, N, K*bits/32]; indices int32 [n_idx];
-    returns bf16 [n_idx, M, N]."""
+    """ops::gather_qmm (mlx-rs/src/ops/quantization.rs:160-230), same argument order and defaults.
+    x: [..., M, K] in bfloat16, float16 or float32 (scales and biases in the same type); w: int32
+    [..., N, K*bits/32] (transpose = False: [..., K, N*bits/32]).  The leading axes of x and of w are
+    batch axes; ``lhs_indices`` / ``rhs_indices`` (int32, any shapes) index the flattened batches and
+    are broadcast against each other; an absent one counts through its batch.  Returns
+    [*broadcast shape, M, N]."""
     lib = load_library()
-    _need(x, torch.bfloat16, "x")
+    dt = _float_dtype(x, "x")
     _need(w, torch.int32, "w")
-    if x.dim() != 3 or w.dim() != 3:
-        raise capi.MoeError("gather_qmm: x must be [batch, M, K] and w [E, N, K*bits/32]")
-    xb, M, K = x.shape
-    E, N = w.shape[0], (w.shape[1] if transpose else w.shape[2] * 32 // bits)
-    if rhs_indices is None:
-        raise capi.MoeError("gather_qmm: rhs_indices is required")
-    n_idx = rhs_indices.numel()
-    y = torch.empty((n_idx, M, N), dtype=torch.bfloat16, device=x.device)
+    _need(scales, x.dtype, "scales")
+    if biases is None:
+        raise capi.MoeError("gather_qmm: biases are required (affine quantisation)")
+    _need(biases, x.dtype, "biases")
+    if x.dim() < 2 or w.dim() < 2:
+        raise capi.MoeError("gather_qmm: x must be [..., M, K] and w [..., N, K*bits/32]")
+    M, K = x.shape[-2:]
+    xb_shape, wb_shape = tuple(x.shape[:-2]), tuple(w.shape[:-2])
+    xb, E = _prod(xb_shape), _prod(wb_shape)
+    N = w.shape[-2] if transpose else w.shape[-1] * 32 // bits
+    kw = w.shape[-1] * 32 // bits if transpose else w.shape[-2]
+    if kw != K:
+        raise capi.MoeError(f"gather_qmm: x has K = {K}, w has K = {kw}")
+    dev = x.device
+
+    def counted(shape):
+        return torch.arange(_prod(shape), dtype=torch.int32, device=dev).reshape(shape)
+
+    lhs = counted(xb_shape) if lhs_indices is None else lhs_indices
+    rhs = counted(wb_shape) if rhs_indices is None else rhs_indices
+    for t, name in ((lhs, "lhs_indices"), (rhs, "rhs_indices")):
+        if t.dtype != torch.int32 or not t.is_cuda:
+            raise capi.MoeError(f"gather_qmm: {name} must be an int32 device tensor")
+    try:
+        lhs_b, rhs_b = torch.broadcast_tensors(lhs, rhs)
+    except RuntimeError as err:
+        raise capi.MoeError(f"gather_qmm: index shapes {tuple(lhs.shape)} and {tuple(rhs.shape)} do not broadcast") from err
+    out_batch = tuple(lhs_b.shape)
+    lhs_f, rhs_f = lhs_b.reshape(-1).contiguous(), rhs_b.reshape(-1).contiguous()
+    n_idx = rhs_f.numel()
+    y = torch.empty((n_idx, M, N), dtype=x.dtype, device=dev)
     need = C.c_size_t()
-    check(lib.mi_moe_gather_qmm_workspace_size(E, n_idx, M, C.byref(need)))
-    ws = _workspace(need.value, x.device)
-    check(lib.mi_moe_gather_qmm(
-        _ptr(x), _ptr(w), _ptr(_need(scales, torch.bfloat16, "scales")),
-        _ptr(None if biases is None else _need(biases, torch.bfloat16, "biases")),
-        _ptr(None if lhs_indices is None else _need(lhs_indices, torch.int32, "lhs_indices")),
-        _ptr(_need(rhs_indices, torch.int32, "rhs_indices")), n_idx, xb, M, N, K, E, int(transpose),
-        group_size, bits, int(sorted_indices), _ptr(y), _ptr(ws), ws.numel(), _stream()))
-    return y
+    check(lib.mi_moe_gather_qmm_workspace_size(min(max(E, 1), 512), n_idx, M, C.byref(need)))
+    ws = _workspace(need.value, dev)
+    check(lib.mi_moe_gather_qmm_typed(
+        _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(lhs_f), _ptr(rhs_f), n_idx, xb, M, N, K, E, int(transpose),
+        group_size, bits, int(sorted_indices), dt, _ptr(y), _ptr(ws), ws.numel(), _stream()))
+    return y.reshape(*out_batch, M, N)
 
 
 def quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4):
     """ops::quantized_matmul (mlx-rs/src/ops/quantization.rs:91-122) the way QuantizedLinear calls
-    it (transpose = true, mlx-rs/src/nn/quantized.rs:363-386): x: bf16 [..., K]; w: int32
-    [N, K*bits/32]; returns bf16 [..., N].  transpose = False (the op's own default): w int32
-    [K, N*bits/32], scales/biases [K, N/group_size], a plain kernel."""
+    it (transpose = true, mlx-rs/src/nn/quantized.rs:363-386): x: [..., K] in bfloat16, float16 or
+    float32 (scales and biases in the same type); w: int32 [N, K*bits/32]; returns [..., N].
+    transpose = False (the op's own default): w int32 [K, N*bits/32], scales/biases [K, N/group_size]."""
     lib = load_library()
-    _need(x, torch.bfloat16, "x")
+    dt = _float_dtype(x, "x")
     _need(w, torch.int32, "w")
+    _need(scales, x.dtype, "scales")
+    _need(biases, x.dtype, "biases")
     if w.dim() != 2 or x.dim() < 1:
         raise capi.MoeError("quantized_matmul: x must be [..., K] and w [N, K*bits/32]")
     K = x.shape[-1]
     N = w.shape[0] if transpose else w.shape[1] * 32 // bits
     x2 = x.reshape(-1, K)
     M = x2.shape[0]
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
     need = C.c_size_t()
     check(lib.mi_moe_quantized_matmul_workspace_size(M, K, bits, C.byref(need)))
     ws = _workspace(need.value, x.device)
-    check(lib.mi_moe_quantized_matmul(_ptr(x2), _ptr(w), _ptr(_need(scales, torch.bfloat16, "scales")),
-                                      _ptr(_need(biases, torch.bfloat16, "biases")), M, N, K,
-                                      1 if transpose else 0, group_size, bits, _ptr(y), _ptr(ws), ws.numel(),
-                                      _stream()))
+    check(lib.mi_moe_quantized_matmul_typed(_ptr(x2), _ptr(w), _ptr(scales), _ptr(biases), M, N, K,
+                                            1 if transpose else 0, group_size, bits, dt, _ptr(y), _ptr(ws),
+                                            ws.numel(), _stream()))
     return y.reshape(*x.shape[:-1], N)
 
 

@@ -13,6 +13,9 @@ pub type mi_moe_handle = *mut mi_moe_s;
 pub const MI_MOE_SCORE_SOFTMAX_THEN_TOPK_RENORM: i32 = 0;
 pub const MI_MOE_SCORE_SOFTMAX_THEN_TOPK: i32 = 1;
 pub const MI_MOE_SCORE_TOPK_THEN_SOFTMAX: i32 = 2;
+pub const MI_MOE_DTYPE_BF16: i32 = 0;
+pub const MI_MOE_DTYPE_F16: i32 = 1;
+pub const MI_MOE_DTYPE_F32: i32 = 2;
 pub const MI_MOE_N_STAGES: usize = 6;
 pub const MI_MOE_N_KERNEL_TIMES: usize = 8;
 pub const MI_MOE_STATIC_SCRATCH_BYTES: usize = 8388608;
@@ -83,14 +86,21 @@ extern "C" {
     pub fn mi_moe_gather_qmm_workspace_size(n_experts: i32, n_idx: i64, M: i32, bytes: *mut usize) -> c_int;
     pub fn mi_moe_gather_qmm(x: *const u16, w: *const u32, scales: *const u16, biases: *const u16, lhs_indices: *const u32, rhs_indices: *const u32, n_idx: i64, x_batch: i64, M: i32, N: i32, K: i32, n_experts: i32, transpose: i32, group_size: i32, bits: i32, sorted_indices: i32, y: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
 
+    pub fn mi_moe_gather_qmm_typed(x: *const c_void, w: *const u32, scales: *const c_void, biases: *const c_void, lhs_indices: *const u32, rhs_indices: *const u32, n_idx: i64, x_batch: i64, M: i32, N: i32, K: i32, n_experts: i32, transpose: i32, group_size: i32, bits: i32, sorted_indices: i32, dtype: i32, y: *mut c_void, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
+
     pub fn mi_moe_quantized_matmul_workspace_size(M: i64, K: i32, bits: i32, bytes: *mut usize) -> c_int;
     pub fn mi_moe_quantized_matmul(x: *const u16, w: *const u32, scales: *const u16, biases: *const u16, M: i64, N: i32, K: i32, transpose: i32, group_size: i32, bits: i32, y: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
+
+    pub fn mi_moe_quantized_matmul_typed(x: *const c_void, w: *const u32, scales: *const c_void, biases: *const c_void, M: i64, N: i32, K: i32, transpose: i32, group_size: i32, bits: i32, dtype: i32, y: *mut c_void, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
 
     pub fn mi_moe_swiglu(gate: *const u16, up: *const u16, n: i64, out: *mut u16, stream: *mut c_void) -> c_int;
     pub fn mi_moe_combine(y: *const u16, scores: *const u16, inv_perm: *const u32, T: i64, top_k: i32, hidden: i32, out: *mut u16, stream: *mut c_void) -> c_int;
 
     pub fn mi_moe_quantize(w: *const f32, rows: i64, cols: i64, group_size: i32, bits: i32, q: *mut u32, scales: *mut u16, biases: *mut u16, stream: *mut c_void) -> c_int;
     pub fn mi_moe_dequantize(q: *const u32, scales: *const u16, biases: *const u16, rows: i64, cols: i64, group_size: i32, bits: i32, w_hat: *mut f32, stream: *mut c_void) -> c_int;
+
+    pub fn mi_moe_quantize_typed(w: *const f32, rows: i64, cols: i64, group_size: i32, bits: i32, dtype: i32, q: *mut u32, scales: *mut c_void, biases: *mut c_void, stream: *mut c_void) -> c_int;
+    pub fn mi_moe_dequantize_typed(q: *const u32, scales: *const c_void, biases: *const c_void, rows: i64, cols: i64, group_size: i32, bits: i32, dtype: i32, w_hat: *mut f32, stream: *mut c_void) -> c_int;
 
     pub fn mi_moe_stream_probe(buf: *const c_void, bytes: usize, sink: *mut u32, stream: *mut c_void) -> c_int;
 

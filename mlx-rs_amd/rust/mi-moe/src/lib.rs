@@ -48,10 +48,33 @@ fn expect_dtype(a: &Array, dt: Dtype, what: &str) -> Result<(), Exception> {
 pub const DEFAULT_GROUP_SIZE: i32 = 64; // mlx-rs/src/ops/quantization.rs:11-13
 pub const DEFAULT_BITS: i32 = 4;
 
+/// The library's code of a floating element type (`mi_moe_dtype`).
+fn float_code(a: &Array, what: &str) -> Result<i32, Exception> {
+    match a.dtype() {
+        Dtype::Bfloat16 => Ok(sys::MI_MOE_DTYPE_BF16),
+        Dtype::Float16 => Ok(sys::MI_MOE_DTYPE_F16),
+        Dtype::Float32 => Ok(sys::MI_MOE_DTYPE_F32),
+        other => Err(Exception::custom(format!("[mi_moe] {what} must be bfloat16, float16 or float32, got {other:?}"))),
+    }
+}
+
+/// An uninitialised array of `shape` in the element type of `like` (a floating type).
+fn empty_like_dtype(like: &Array, shape: &[i32]) -> Result<Array, Exception> {
+    let a = match like.dtype() {
+        Dtype::Float32 => Array::zeros::<f32>(shape)?,
+        Dtype::Float16 => Array::zeros::<half::f16>(shape)?,
+        _ => Array::zeros::<half::bf16>(shape)?,
+    };
+    a.eval()?;
+    Ok(a)
+}
+
 pub mod ops {
     use super::*;
 
-    /// `(w_q, scales, biases)` of a `[rows, cols]` float32 matrix: `mi_moe_quantize`.
+    /// `(w_q, scales, biases)` of a `[rows, cols]` float32 matrix: `mi_moe_quantize_typed`.  Scales
+    /// and biases come out in float32, the type of the input, as `ops::quantize` gives them
+    /// (`mlx-rs/src/ops/quantization.rs:50-83`); cast them for a bfloat16 model.
     pub fn quantize<D: DeviceAccess>(
         w: &Array,
         group_size: impl Into<Option<i32>>,
@@ -64,18 +87,18 @@ pub mod ops {
         w.eval()?;
         let (rows, cols) = (w.dim(-2) as i64, w.dim(-1) as i64);
         let mut q = Array::zeros::<u32>(&[rows as i32, (cols * bits as i64 / 32) as i32])?;
-        let mut s = Array::zeros::<half::bf16>(&[rows as i32, (cols / group_size as i64) as i32])?;
-        let mut b = Array::zeros::<half::bf16>(&[rows as i32, (cols / group_size as i64) as i32])?;
+        let mut s = Array::zeros::<f32>(&[rows as i32, (cols / group_size as i64) as i32])?;
+        let mut b = Array::zeros::<f32>(&[rows as i32, (cols / group_size as i64) as i32])?;
         q.eval()?;
         s.eval()?;
         b.eval()?;
         check(unsafe {
-            sys::mi_moe_quantize(D::device_ptr(w) as *const f32, rows, cols, group_size, bits, D::device_ptr_mut(&mut q) as *mut u32, D::device_ptr_mut(&mut s) as *mut u16, D::device_ptr_mut(&mut b) as *mut u16, D::hip_stream(stream))
+            sys::mi_moe_quantize_typed(D::device_ptr(w) as *const f32, rows, cols, group_size, bits, sys::MI_MOE_DTYPE_F32, D::device_ptr_mut(&mut q) as *mut u32, D::device_ptr_mut(&mut s), D::device_ptr_mut(&mut b), D::hip_stream(stream))
         })?;
         Ok((q, s, b))
     }
 
-    /// `mi_moe_dequantize`: float32 `[rows, cols]`.
+    /// `mi_moe_dequantize_typed`: float32 `[rows, cols]`; scales and biases in any floating type.
     pub fn dequantize<D: DeviceAccess>(
         w: &Array,
         scales: &Array,
@@ -87,20 +110,21 @@ pub mod ops {
         let group_size = group_size.into().unwrap_or(DEFAULT_GROUP_SIZE);
         let bits = bits.into().unwrap_or(DEFAULT_BITS);
         expect_dtype(w, Dtype::Uint32, "w")?;
-        expect_dtype(scales, Dtype::Bfloat16, "scales")?;
-        expect_dtype(biases, Dtype::Bfloat16, "biases")?;
+        let dt = float_code(scales, "scales")?;
+        expect_dtype(biases, scales.dtype(), "biases")?;
         let rows = w.dim(-2) as i64;
         let cols = w.dim(-1) as i64 * 32 / bits as i64;
         let mut out = Array::zeros::<f32>(&[rows as i32, cols as i32])?;
         out.eval()?;
         check(unsafe {
-            sys::mi_moe_dequantize(D::device_ptr(w) as *const u32, D::device_ptr(scales) as *const u16, D::device_ptr(biases) as *const u16, rows, cols, group_size, bits, D::device_ptr_mut(&mut out) as *mut f32, D::hip_stream(stream))
+            sys::mi_moe_dequantize_typed(D::device_ptr(w) as *const u32, D::device_ptr(scales), D::device_ptr(biases), rows, cols, group_size, bits, dt, D::device_ptr_mut(&mut out) as *mut f32, D::hip_stream(stream))
         })?;
         Ok(out)
     }
 
-    /// `x [M, K]` times one quantized matrix; `transpose` defaults to `true` as in
-    /// `quantized_matmul` (`mlx-rs/src/ops/quantization.rs:91-122`).
+    /// `x [..., K]` times one quantized matrix, in any floating type (scales and biases in the type
+    /// of `x`); `transpose` defaults to `false` as in `quantized_matmul`
+    /// (`mlx-rs/src/ops/quantization.rs:91-122`).
     #[allow(clippy::too_many_arguments)]
     pub fn quantized_matmul<D: DeviceAccess>(
         x: &Array,
@@ -112,11 +136,13 @@ pub mod ops {
         bits: impl Into<Option<i32>>,
         stream: &Stream,
     ) -> Result<Array, Exception> {
-        let transpose = transpose.into().unwrap_or(true);
+        let transpose = transpose.into().unwrap_or(false);
         let group_size = group_size.into().unwrap_or(DEFAULT_GROUP_SIZE);
         let bits = bits.into().unwrap_or(DEFAULT_BITS);
-        expect_dtype(x, Dtype::Bfloat16, "x")?;
+        let dt = float_code(x, "x")?;
         expect_dtype(w, Dtype::Uint32, "w")?;
+        expect_dtype(scales, x.dtype(), "scales")?;
+        expect_dtype(biases, x.dtype(), "biases")?;
         let k = x.dim(-1);
         let m: i64 = x.shape()[..x.ndim() - 1].iter().map(|&d| d as i64).product();
         let n = if transpose { w.dim(-2) } else { w.dim(-1) * 32 / bits };
@@ -125,25 +151,26 @@ pub mod ops {
         let mut ws = D::device_buffer(ws_bytes.max(256))?;
         let mut shape = x.shape().to_vec();
         *shape.last_mut().unwrap() = n;
-        let mut y = Array::zeros::<half::bf16>(&shape)?;
-        y.eval()?;
+        let mut y = empty_like_dtype(x, &shape)?;
         check(unsafe {
-            sys::mi_moe_quantized_matmul(D::device_ptr(x) as *const u16, D::device_ptr(w) as *const u32, D::device_ptr(scales) as *const u16, D::device_ptr(biases) as *const u16, m, n, k, transpose as i32, group_size, bits, D::device_ptr_mut(&mut y) as *mut u16, D::device_ptr_mut(&mut ws), ws_bytes, D::hip_stream(stream))
+            sys::mi_moe_quantized_matmul_typed(D::device_ptr(x), D::device_ptr(w) as *const u32, D::device_ptr(scales), D::device_ptr(biases), m, n, k, transpose as i32, group_size, bits, dt, D::device_ptr_mut(&mut y), D::device_ptr_mut(&mut ws), ws_bytes, D::hip_stream(stream))
         })?;
         Ok(y)
     }
 
-    /// `gather_qmm` with the argument list of `mlx-rs/src/ops/quantization.rs:180-230`.
-    /// `x`: bf16 `[batch, M, K]`; `w`: `[E, N, K*bits/32]`; `rhs_indices` is required here
-    /// (every switch layer passes it), `lhs_indices = None` pairs row `j` with index `j`.
+    /// `gather_qmm` with the argument list and the batch semantics of
+    /// `mlx-rs/src/ops/quantization.rs:160-230`: `x` is `[..., M, K]` in any floating type, `w`
+    /// `[..., N, K*bits/32]`; the index arrays (any shapes) address the flattened leading axes and
+    /// are broadcast against each other; an absent one counts through its batch.  Returns
+    /// `[*broadcast shape, M, N]`.
     #[allow(clippy::too_many_arguments)]
-    pub fn gather_qmm<'l, D: DeviceAccess>(
+    pub fn gather_qmm<'l, 'r, D: DeviceAccess>(
         x: &Array,
         w: &Array,
         scales: &Array,
         biases: &Array,
         lhs_indices: impl Into<Option<&'l Array>>,
-        rhs_indices: &Array,
+        rhs_indices: impl Into<Option<&'r Array>>,
         transpose: impl Into<Option<bool>>,
         group_size: impl Into<Option<i32>>,
         bits: impl Into<Option<i32>>,
@@ -154,25 +181,47 @@ pub mod ops {
         let group_size = group_size.into().unwrap_or(DEFAULT_GROUP_SIZE);
         let bits = bits.into().unwrap_or(DEFAULT_BITS);
         let sorted = sorted_indices.into().unwrap_or(false);
-        let lhs = lhs_indices.into();
-        expect_dtype(x, Dtype::Bfloat16, "x")?;
+        let dt = float_code(x, "x")?;
         expect_dtype(w, Dtype::Uint32, "w")?;
-        expect_dtype(rhs_indices, Dtype::Uint32, "rhs_indices")?;
-        if x.ndim() != 3 || w.ndim() != 3 {
-            return Err(Exception::custom("[mi_moe] gather_qmm takes x [batch, M, K] and w [E, N, K*bits/32]"));
+        expect_dtype(scales, x.dtype(), "scales")?;
+        expect_dtype(biases, x.dtype(), "biases")?;
+        if x.ndim() < 2 || w.ndim() < 2 {
+            return Err(Exception::custom("[mi_moe] gather_qmm takes x [..., M, K] and w [..., N, K*bits/32]"));
         }
-        let (x_batch, m, k) = (x.dim(0) as i64, x.dim(1), x.dim(2));
-        let e = w.dim(0);
-        let n = if transpose { w.dim(1) } else { w.dim(2) * 32 / bits };
-        let n_idx = rhs_indices.size() as i64;
+        let (m, k) = (x.dim(-2), x.dim(-1));
+        let x_batch_shape = &x.shape()[..x.ndim() - 2];
+        let w_batch_shape = &w.shape()[..w.ndim() - 2];
+        let x_batch: i64 = x_batch_shape.iter().map(|&d| d as i64).product();
+        let e: i64 = w_batch_shape.iter().map(|&d| d as i64).product();
+        let n = if transpose { w.dim(-2) } else { w.dim(-1) * 32 / bits };
+        // an absent index array counts through its batch, in the batch's shape
+        let counted = |count: i64, shape: &[i32]| -> Result<Array, Exception> {
+            Array::arange::<_, u32>(None, count, None)?.reshape(shape)
+        };
+        let lhs = match lhs_indices.into() {
+            Some(a) => a.as_dtype(Dtype::Uint32)?,
+            None => counted(x_batch, x_batch_shape)?,
+        };
+        let rhs = match rhs_indices.into() {
+            Some(a) => a.as_dtype(Dtype::Uint32)?,
+            None => counted(e, w_batch_shape)?,
+        };
+        let both = mlx_rs::ops::broadcast_arrays(&[&lhs, &rhs])?;
+        let batch_shape = both[0].shape().to_vec();
+        let lhs = both[0].flatten(None, None)?;
+        let rhs = both[1].flatten(None, None)?;
+        lhs.eval()?; // (materialised, row-major contiguous)
+        rhs.eval()?;
+        let n_idx = rhs.size() as i64;
         let mut ws_bytes = 0usize;
-        check(unsafe { sys::mi_moe_gather_qmm_workspace_size(e, n_idx, m, &mut ws_bytes) })?;
+        check(unsafe { sys::mi_moe_gather_qmm_workspace_size(e.clamp(1, 512) as i32, n_idx, m, &mut ws_bytes) })?;
         let mut ws = D::device_buffer(ws_bytes.max(256))?;
-        let mut y = Array::zeros::<half::bf16>(&[n_idx as i32, m, n])?;
-        y.eval()?;
-        let lhs_ptr = lhs.map(|a| D::device_ptr(a) as *const u32).unwrap_or(std::ptr::null());
+        let mut shape = batch_shape;
+        shape.push(m);
+        shape.push(n);
+        let mut y = empty_like_dtype(x, &shape)?;
         check(unsafe {
-            sys::mi_moe_gather_qmm(D::device_ptr(x) as *const u16, D::device_ptr(w) as *const u32, D::device_ptr(scales) as *const u16, D::device_ptr(biases) as *const u16, lhs_ptr, D::device_ptr(rhs_indices) as *const u32, n_idx, x_batch, m, n, k, e, transpose as i32, group_size, bits, sorted as i32, D::device_ptr_mut(&mut y) as *mut u16, D::device_ptr_mut(&mut ws), ws_bytes, D::hip_stream(stream))
+            sys::mi_moe_gather_qmm_typed(D::device_ptr(x), D::device_ptr(w) as *const u32, D::device_ptr(scales), D::device_ptr(biases), D::device_ptr(&lhs) as *const u32, D::device_ptr(&rhs) as *const u32, n_idx, x_batch, m, n, k, e as i32, transpose as i32, group_size, bits, sorted as i32, dt, D::device_ptr_mut(&mut y), D::device_ptr_mut(&mut ws), ws_bytes, D::hip_stream(stream))
         })?;
         Ok(y)
     }

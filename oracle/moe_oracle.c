@@ -488,7 +488,7 @@ static int moe_forward_impl(const orc_config *cfg, const orc_weights *w, const u
                             int n_threads, const uint16_t *residual) {
   const int H = cfg->hidden, E = cfg->n_experts, k = cfg->top_k, I = cfg->intermediate;
   const int bits = cfg->bits, group = cfg->group_size;
-  if (!(bits == 4 || bits == 8)) return fail("forward: bits must be 4 or 8");
+  if (!(bits == 2 || bits == 4 || bits == 8)) return fail("forward: bits must be 2, 4 or 8");
   if (group != 64 && group != 32 && group != 128) return fail("forward: unsupported group_size");
   if (H % group || I % group) return fail("forward: hidden and intermediate must be divisible by group_size");
   if (k < 1 || k > E) return fail("forward: top_k must be in [1, n_experts]");

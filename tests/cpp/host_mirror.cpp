@@ -48,8 +48,9 @@ static int run_errors() {
   Array w = Array::from_device_ptr(nullptr, {2, 16, 16}, Dtype::Uint32);
   Array s = Array::from_device_ptr(nullptr, {2, 16, 2}, Dtype::Bfloat16);
   Array idx = Array::from_device_ptr(nullptr, {4}, Dtype::Uint32);
-  auto r1 = ops::gather_qmm(x, w, s, &s, nullptr, nullptr);
-  EXPECT(r1.is_err() && contains(r1.error(), "rhs_indices"));
+  Array bad_idx = Array::from_device_ptr(nullptr, {4}, Dtype::Float32);
+  auto r1 = ops::gather_qmm(x, w, s, &s, nullptr, &bad_idx);
+  EXPECT(r1.is_err() && contains(r1.error(), "uint32"));
   auto r2 = ops::gather_qmm(x, w, s, nullptr, nullptr, &idx);
   EXPECT(r2.is_err() && contains(r2.error(), "biases"));
   auto r3 = ops::gather_qmm(w, w, s, &s, nullptr, &idx);
@@ -133,8 +134,26 @@ static int run_forward(const std::string &dir) {
   dump(dir + "/gq.bin", g);
   // library-side refusal surfaces as an error value with its text
   auto bad2 = ops::gather_qmm(x.reshape({T, 1, H}), gate.weight, gate.scales, &gate.biases, &lhs, &rhs,
-                              true, 32, (int32_t)bits, false);
+                              true, 48, (int32_t)bits, false);
   EXPECT(bad2.is_err() && contains(bad2.error(), "group_size"));
+  // index arrays of shapes [2, 1] and [1, 3] broadcast to [2, 3]: the same bytes as the six pairs spelt out
+  {
+    const uint32_t l21[2] = {5, 1}, r13[3] = {3, 0, 2}, l6[6] = {5, 5, 5, 1, 1, 1}, r6[6] = {3, 0, 2, 3, 0, 2};
+    Array a21 = Array::from_host(l21, {2, 1}, Dtype::Uint32).unwrap(), a13 = Array::from_host(r13, {1, 3}, Dtype::Uint32).unwrap();
+    Array a6 = Array::from_host(l6, {6}, Dtype::Uint32).unwrap(), b6 = Array::from_host(r6, {6}, Dtype::Uint32).unwrap();
+    Array yb = ops::gather_qmm(x.reshape({T, 1, H}), gate.weight, gate.scales, &gate.biases, &a21, &a13, true, 64,
+                               (int32_t)bits, false).unwrap();
+    Array yf = ops::gather_qmm(x.reshape({T, 1, H}), gate.weight, gate.scales, &gate.biases, &a6, &b6, true, 64,
+                               (int32_t)bits, false).unwrap();
+    EXPECT(yb.ndim() == 4 && yb.dim(0) == 2 && yb.dim(1) == 3 && yb.dim(2) == 1 && yb.dim(3) == I);
+    std::vector<uint16_t> hb((size_t)yb.size()), hf((size_t)yf.size());
+    yb.to_host(hb.data()).unwrap();
+    yf.to_host(hf.data()).unwrap();
+    EXPECT(hb.size() == hf.size() && hb == hf);
+    auto bad3 = ops::gather_qmm(x.reshape({T, 1, H}), gate.weight, gate.scales, &gate.biases, &a6, &a13, true, 64,
+                                (int32_t)bits, false);
+    EXPECT(bad3.is_err() && contains(bad3.error(), "broadcast"));
+  }
 
   // ops::quantize / ops::dequantize with the defaults (group 64, 4 bits)
   Array wf = load(dir, "wf.bin", {qrows, qcols}, Dtype::Float32);

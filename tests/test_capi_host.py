@@ -41,7 +41,7 @@ def cfg(**kw):
 
 
 @pytest.mark.parametrize("kw,needle", [
-    (dict(hidden=100), "hidden"), (dict(bits=3), "bits"), (dict(group_size=32), "group_size"),
+    (dict(hidden=100), "hidden"), (dict(bits=3), "bits"), (dict(group_size=48), "group_size"), (dict(group_size=128, hidden=192), "group_size"),
     (dict(top_k=9), "top_k"), (dict(top_k=0), "top_k"), (dict(n_experts=0), "n_experts"),
     (dict(intermediate=96), "intermediate"), (dict(score_mode=7), "score_mode"),
     (dict(hidden=192), "128"),
@@ -78,7 +78,7 @@ def test_null_and_range_checks(lib):
     assert lib.mi_moe_dispatch(None, 8, 4, None, None, None, None, None, 0, None) != 0
     assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 96, 64, 3, 0, 64, 4, 0,
                                  None, None, 0, None) != 0
-    assert "transpose" in m.capi.last_error()      # untransposed weights need N to be a multiple of 64
+    assert "group_size" in m.capi.last_error()     # untransposed weights are quantised along N: N % group_size
     assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 64, 64, 3, 1, 64, 5, 0,
                                  None, None, 0, None) != 0
     assert "bits" in m.capi.last_error()
@@ -95,9 +95,12 @@ def test_null_and_range_checks(lib):
     assert lib.mi_moe_quantized_matmul_workspace_size(-1, 128, 4, C.byref(n2)) != 0 and n2.value == 7
     assert lib.mi_moe_quantized_matmul_workspace_size(300, 256, 4, C.byref(n2)) == 0 and n2.value > 300 * 256 * 2
     assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 96, 128, 0, 64, 4, None, None, 0, None) != 0
-    assert "transpose" in m.capi.last_error()
-    assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 60, 128, 1, 64, 4, None, None, 0, None) != 0
-    assert "N must" in m.capi.last_error()
+    assert "group_size" in m.capi.last_error()
+    assert lib.mi_moe_quantized_matmul(None, None, None, None, 4, 64, 100, 1, 32, 4, None, None, 0, None) != 0
+    assert "K (100)" in m.capi.last_error()
+    assert lib.mi_moe_quantized_matmul_typed(None, None, None, None, 4, 64, 128, 1, 64, 4, 3, None, None, 0, None) != 0
+    assert "dtype" in m.capi.last_error()
+    assert lib.mi_moe_quantize_typed(None, 2, 128, 64, 4, 9, None, None, None, None) != 0 and "dtype" in m.capi.last_error()
     assert lib.mi_moe_quantized_matmul(None, None, None, None, 0, 64, 128, 1, 64, 4, None, None, 0, None) == 0
     assert lib.mi_moe_rms_norm(None, None, 1e-5, 4, 100, None, None) != 0 and "hidden" in m.capi.last_error()
     assert lib.mi_moe_rms_norm(None, None, -1.0, 4, 128, None, None) != 0 and "eps" in m.capi.last_error()

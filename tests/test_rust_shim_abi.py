@@ -65,7 +65,7 @@ def parse_header():
             for nm in mm.group(2).split(","):
                 fields.append((nm.strip(), ty))
         structs[m.group(2)] = fields
-    consts = {m.group(1): int(m.group(2)) for m in re.finditer(r"(MI_MOE_SCORE_\w+)\s*=\s*(\d+)", src)}
+    consts = {m.group(1): int(m.group(2)) for m in re.finditer(r"(MI_MOE_(?:SCORE|DTYPE)_\w+)\s*=\s*(\d+)", src)}
     consts.update({m.group(1): int(m.group(2)) for m in re.finditer(r"#define\s+(MI_MOE_N_STAGES|MI_MOE_N_KERNEL_TIMES|MI_MOE_STATIC_SCRATCH_BYTES)\s+(\d+)", src)})
     return funcs, structs, consts
 
@@ -94,7 +94,7 @@ def parse_rust():
 def test_every_header_function_is_declared_identically():
     hf, _, _ = parse_header()
     rf, _, _ = parse_rust()
-    assert len(hf) == 24, sorted(hf)
+    assert len(hf) == 28, sorted(hf)
     assert sorted(hf) == sorted(rf)
     for name, (ret, args) in hf.items():
         assert rf[name][0] == ret, (name, rf[name][0], ret)
@@ -112,7 +112,7 @@ def test_structs_have_the_same_fields_in_the_same_order():
 def test_constants_agree():
     _, _, hc = parse_header()
     _, _, rc = parse_rust()
-    assert len(hc) == 6
+    assert len(hc) == 9
     assert hc == rc
 
 

@@ -34,13 +34,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # inside this script: the figure is carried from the named file under profiles/, it is not measured by this run.
 CARRIED_TRAFFIC = {
     "decode": (1.976e8, "profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt"),
-    "prefill": (5.50e8, "profiles/qmm_large_kernel_prefill_tokens4096_counters.txt"),
-    "mixtral_decode": (2.530e8, "profiles/qmm_small_kernel_decode_mixtral_batch1.txt"),
+    "prefill": (4.048e8, "profiles/qmm_large_kernel_prefill_tokens4096_counters.txt"),
+    "mixtral_decode": (2.529e8, "profiles/qmm_small_kernel_decode_mixtral_batch1.txt"),
 }
 
 WORKLOADS = {
     # name: (config key, batches, headline batch, zipf s, bound)
     "decode": ("qwen3_30b_a3b", [1, 8, 32], 32, None, "hbm"),
+    "decode_batch1": ("qwen3_30b_a3b", [1], 1, None, "hbm"),   # one batch per process: for per-kernel profiles
+    "decode_batch8": ("qwen3_30b_a3b", [8], 8, None, "hbm"),
     "prefill": ("qwen3_30b_a3b", [4096], 4096, 1.1, "mfma"),
     "mixtral_decode": ("mixtral_8x7b", [1], 1, None, "hbm"),
     "mixtral_prefill": ("mixtral_8x7b", [2048], 2048, None, "mfma"),

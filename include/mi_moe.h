@@ -197,6 +197,10 @@ int mi_moe_dispatch(const uint32_t *expert_of_pair, int64_t P, int32_t n_experts
  * quantised along N), group sizes 32 and 128, 2-bit codes -- is served by plain kernels that need no
  * workspace and no alignment.
  * sorted_indices is a hint, results do not depend on it.
+ * Index values live in device memory and cannot be checked by the call: an lhs index beyond
+ * x_batch - 1 or an rhs index beyond n_experts - 1 is clamped to the last matrix by the kernels (the
+ * output rows it belongs to are then meaningless, but nothing outside the operands is read).
+ * x_batch = 0 means "not told" (no clamp on lhs); without lhs_indices, n_idx may not exceed x_batch.
  * workspace >= mi_moe_gather_qmm_workspace_size. */
 int mi_moe_gather_qmm_workspace_size(int32_t n_experts, int64_t n_idx, int32_t M, size_t *bytes);
 int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scales,

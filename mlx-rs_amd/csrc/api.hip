@@ -364,13 +364,13 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     // the sorted order belongs to pair perm[r], token src_of[r], expert topk_idx[perm[r]].
     const size_t PI = (size_t)P * c.intermediate;
     MI_HIP(launch_qmm_plain(x, h->w.gate.w, h->w.gate.scales, h->w.gate.biases, f.src_of, f.topk_idx, f.perm, nullptr,
-                            P, 1, c.intermediate, c.hidden, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.gu, st));
-    MI_HIP(launch_qmm_plain(x, h->w.up.w, h->w.up.scales, h->w.up.biases, f.src_of, f.topk_idx, f.perm, nullptr, P, 1,
-                            c.intermediate, c.hidden, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.gu + PI, st));
+                            (uint32_t)T, (uint32_t)c.n_experts, P, 1, c.intermediate, c.hidden, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.gu, st));
+    MI_HIP(launch_qmm_plain(x, h->w.up.w, h->w.up.scales, h->w.up.biases, f.src_of, f.topk_idx, f.perm, nullptr,
+                            (uint32_t)T, (uint32_t)c.n_experts, P, 1, c.intermediate, c.hidden, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.gu + PI, st));
     MI_HIP(launch_swiglu(f.gu, f.gu + PI, (int64_t)PI, f.hh, st));
     MI_STAGE_DONE();
     MI_HIP(launch_qmm_plain(f.hh, h->w.down.w, h->w.down.scales, h->w.down.biases, nullptr, f.topk_idx, f.perm, f.perm,
-                            P, 1, c.hidden, c.intermediate, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.y, st));
+                            0u, (uint32_t)c.n_experts, P, 1, c.hidden, c.intermediate, c.group_size, c.bits, true, MI_MOE_DTYPE_BF16, f.y, st));
     MI_STAGE_DONE();
   } else if (large_qmm_applies(a) && !ev) {
     // Four chains that share no rows: the three tile classes and the streamed segments, each
@@ -653,8 +653,8 @@ static int check_qmm_shape(const char *who, int32_t dtype, int32_t transpose, in
 }
 
 static int gather_qmm_impl(const void *x, const uint32_t *w, const void *scales, const void *biases,
-                           const uint32_t *lhs_indices, const uint32_t *rhs_indices, int64_t n_idx, int32_t M,
-                           int32_t N, int32_t K, int32_t n_experts, int32_t transpose, int32_t group_size,
+                           const uint32_t *lhs_indices, const uint32_t *rhs_indices, int64_t n_idx, int64_t x_batch,
+                           int32_t M, int32_t N, int32_t K, int32_t n_experts, int32_t transpose, int32_t group_size,
                            int32_t bits, int32_t dtype, void *y, void *workspace, size_t workspace_bytes,
                            void *stream) {
   if (check_qmm_shape("gather_qmm", dtype, transpose, group_size, bits, N, K)) return 1;
@@ -664,10 +664,18 @@ static int gather_qmm_impl(const void *x, const uint32_t *w, const void *scales,
   if (n_idx == 0) return 0;
   if (!x || !w || !scales || !biases || !y) return fail("gather_qmm: x, w, scales, biases and y must be non-NULL");
   if (!rhs_indices) return fail("gather_qmm: rhs_indices is required");
+  // x_batch = matrices in x (0 = not told).  Without lhs_indices index j reads x[j], so there must be n_idx of them;
+  // with lhs_indices the kernels clamp an index beyond x_batch - 1 (and an expert index beyond n_experts - 1) instead
+  // of following it: the rows it belongs to are then meaningless, but no memory outside the operands is read.
+  if (x_batch < 0 || x_batch > (int64_t)UINT32_MAX) return fail("gather_qmm: x_batch out of range");
+  if (!lhs_indices && x_batch > 0 && n_idx > x_batch)
+    return fail("gather_qmm: %lld indices without lhs_indices need as many matrices in x, got %lld", (long long)n_idx,
+                (long long)x_batch);
+  const uint32_t n_lhs = (uint32_t)x_batch;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (!tuned_shape(dtype, transpose, group_size, bits, N, K) || n_experts > 512) {  // the plain kernels, no workspace
-    MI_HIP(launch_qmm_plain(x, w, scales, biases, lhs_indices, rhs_indices, nullptr, nullptr, n_idx * M, M, N, K,
-                            group_size, bits, transpose != 0, dtype, y, st));
+    MI_HIP(launch_qmm_plain(x, w, scales, biases, lhs_indices, rhs_indices, nullptr, nullptr, n_lhs, (uint32_t)n_experts,
+                            n_idx * M, M, N, K, group_size, bits, transpose != 0, dtype, y, st));
     return 0;
   }
   if (!aligned16(x) || !aligned16(w) || !aligned16(scales) || !aligned16(biases) || !aligned16(y))
@@ -686,7 +694,7 @@ static int gather_qmm_impl(const void *x, const uint32_t *w, const void *scales,
   uint32_t *dst_rows = cv.take<uint32_t>((size_t)rows);
   MI_HIP(launch_dispatch(rhs_indices, n_idx, n_experts, 1, counts, offsets, perm, nullptr, nullptr, work,
                          nullptr, 0, 0, scratch, st));
-  MI_HIP(launch_row_maps(perm, lhs_indices, offsets, n_idx, M, n_experts, src_rows, dst_rows, work, st));
+  MI_HIP(launch_row_maps(perm, lhs_indices, n_lhs, offsets, n_idx, M, n_experts, src_rows, dst_rows, work, st));
   GroupedArgs a{};
   a.x = static_cast<const uint16_t *>(x);
   a.src_rows = src_rows;
@@ -710,8 +718,7 @@ int mi_moe_gather_qmm(const uint16_t *x, const uint32_t *w, const uint16_t *scal
                       int32_t transpose, int32_t group_size, int32_t bits, int32_t sorted_indices,
                       uint16_t *y, void *workspace, size_t workspace_bytes, void *stream) try {
   (void)sorted_indices;  // a hint in MLX; the segments are rebuilt here either way
-  (void)x_batch;
-  return gather_qmm_impl(x, w, scales, biases, lhs_indices, rhs_indices, n_idx, M, N, K, n_experts, transpose,
+  return gather_qmm_impl(x, w, scales, biases, lhs_indices, rhs_indices, n_idx, x_batch, M, N, K, n_experts, transpose,
                          group_size, bits, MI_MOE_DTYPE_BF16, y, workspace, workspace_bytes, stream);
 } MI_CATCH("gather_qmm")
 
@@ -721,8 +728,7 @@ int mi_moe_gather_qmm_typed(const void *x, const uint32_t *w, const void *scales
                             int32_t transpose, int32_t group_size, int32_t bits, int32_t sorted_indices,
                             int32_t dtype, void *y, void *workspace, size_t workspace_bytes, void *stream) try {
   (void)sorted_indices;
-  (void)x_batch;
-  return gather_qmm_impl(x, w, scales, biases, lhs_indices, rhs_indices, n_idx, M, N, K, n_experts, transpose,
+  return gather_qmm_impl(x, w, scales, biases, lhs_indices, rhs_indices, n_idx, x_batch, M, N, K, n_experts, transpose,
                          group_size, bits, dtype, y, workspace, workspace_bytes, stream);
 } MI_CATCH("gather_qmm_typed")
 
@@ -752,7 +758,7 @@ static int quantized_matmul_impl(const void *x, const uint32_t *w, const void *s
   if (!x || !w || !scales || !biases || !y) return fail("quantized_matmul: x, w, scales, biases and y must be non-NULL");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (!tuned_shape(dtype, transpose, group_size, bits, N, K)) {  // the plain kernels, no workspace
-    MI_HIP(launch_qmm_plain(x, w, scales, biases, nullptr, nullptr, nullptr, nullptr, M, 1, N, K, group_size, bits,
+    MI_HIP(launch_qmm_plain(x, w, scales, biases, nullptr, nullptr, nullptr, nullptr, 0u, 1u, M, 1, N, K, group_size, bits,
                             transpose != 0, dtype, y, st));
     return 0;
   }

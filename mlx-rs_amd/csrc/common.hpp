@@ -250,7 +250,7 @@ bool large_qmm_applies(const GroupedArgs &a);
 hipError_t launch_large_qmm_class(const GroupedArgs &a, bool glu, int cls, hipStream_t st);
 hipError_t launch_small_qmm(const GroupedArgs &a, bool glu, hipStream_t st);
 hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *out, hipStream_t st);
-hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
+hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, uint32_t n_lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
                            uint32_t *work, hipStream_t st);
 hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t *mtiles, int cap256,
@@ -265,11 +265,12 @@ hipError_t launch_rms_norm(const uint16_t *x, const uint16_t *weight, float eps,
                            uint16_t *out, hipStream_t st);
 // plain products (any float type, group sizes 32 / 64 / 128, 2 / 4 / 8 bits, both weight layouts);
 // dt: 0 bf16, 1 fp16, 2 fp32.  Output row r = j * M + m: expert rhs[rhs_map ? rhs_map[j] : j] (0 without
-// rhs), x row (lhs ? lhs[j] : j) * M + m, destination row dst_map ? dst_map[r] : r.
+// rhs), x row (lhs ? lhs[j] : j) * M + m, destination row dst_map ? dst_map[r] : r.  n_lhs / n_rhs: how many
+// matrices the lhs / rhs indices may address (0 = unknown); an index beyond is clamped to the last one.
 hipError_t launch_qmm_plain(const void *x, const uint32_t *w, const void *scales, const void *biases,
                             const uint32_t *lhs, const uint32_t *rhs, const uint32_t *rhs_map,
-                            const uint32_t *dst_map, int64_t rows, int M, int N, int K, int group, int bits,
-                            bool transpose, int dt, void *y, hipStream_t st);
+                            const uint32_t *dst_map, uint32_t n_lhs, uint32_t n_rhs, int64_t rows, int M, int N,
+                            int K, int group, int bits, bool transpose, int dt, void *y, hipStream_t st);
 hipError_t launch_quantize(const float *w, int64_t rows, int64_t cols, int group, int bits,
                            uint32_t *q, void *s, void *b, int dt, hipStream_t st);
 hipError_t launch_dequantize(const uint32_t *q, const void *s, const void *b,

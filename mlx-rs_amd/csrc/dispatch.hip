@@ -163,7 +163,7 @@ hipError_t launch_dense_records(int64_t M, int big_thr, uint32_t *work, uint32_t
 
 // Row maps for the stand-alone gather_qmm: sorted position q of index j = perm[q]
 // covers M rows; x rows come from lhs[j]*M + m, outputs go to j*M + m.
-__global__ void row_maps_kernel(const uint32_t *__restrict__ perm, const uint32_t *__restrict__ lhs,
+__global__ void row_maps_kernel(const uint32_t *__restrict__ perm, const uint32_t *__restrict__ lhs, uint32_t n_lhs,
                                 const uint32_t *__restrict__ offsets, int64_t n_idx, int M, int E,
                                 uint32_t *__restrict__ src_rows, uint32_t *__restrict__ dst_rows,
                                 uint32_t *__restrict__ work) {
@@ -177,15 +177,17 @@ __global__ void row_maps_kernel(const uint32_t *__restrict__ perm, const uint32_
   const int64_t q = i / M;
   const int m = (int)(i % M);
   const uint32_t j = perm[q];
-  src_rows[i] = (lhs ? lhs[j] : j) * (uint32_t)M + m;
+  uint32_t xb = lhs ? lhs[j] : j;
+  if (n_lhs && xb >= n_lhs) xb = n_lhs - 1u;  // an index past x's batch is clamped, never followed
+  src_rows[i] = xb * (uint32_t)M + m;
   dst_rows[i] = j * (uint32_t)M + m;
 }
 
-hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, const uint32_t *offsets,
+hipError_t launch_row_maps(const uint32_t *perm, const uint32_t *lhs, uint32_t n_lhs, const uint32_t *offsets,
                            int64_t n_idx, int M, int E, uint32_t *src_rows, uint32_t *dst_rows,
                            uint32_t *work, hipStream_t st) {
   int64_t n = n_idx * M > E ? n_idx * M : E;
-  row_maps_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(perm, lhs, offsets, n_idx, M, E,
+  row_maps_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(perm, lhs, n_lhs, offsets, n_idx, M, E,
                                                               src_rows, dst_rows, work);
   return hipGetLastError();
 }

@@ -133,7 +133,10 @@ hipError_t launch_dequantize(const uint32_t *q, const void *s, const void *b,
 //   destination row = dst_map ? dst_map[r] : r.
 struct PlainMaps {
   const uint32_t *lhs, *rhs, *rhs_map, *dst_map;
+  uint32_t n_lhs, n_rhs;  // matrices behind lhs / rhs (0 = unknown): indices beyond are clamped, never followed
 };
+
+__device__ __forceinline__ int64_t clamped_index(uint32_t v, uint32_t n) { return n && v >= n ? n - 1u : v; }
 
 // transpose = true: w [E, N, K*bits/32], scales / biases [E, N, K/group].  One wave per output
 // element, lanes over the packed words of the weight row, sum over the lanes in a fixed order.
@@ -149,8 +152,8 @@ __global__ __launch_bounds__(256) void qmm_plain_t_kernel(const T *__restrict__ 
   const int lane = lane_id();
   const int64_t j = r / M;
   const int m = (int)(r % M);
-  const int64_t e = mp.rhs ? (int64_t)mp.rhs[mp.rhs_map ? mp.rhs_map[j] : j] : 0;
-  const int64_t xb = mp.lhs ? (int64_t)mp.lhs[j] : j;
+  const int64_t e = mp.rhs ? clamped_index(mp.rhs[mp.rhs_map ? mp.rhs_map[j] : j], mp.n_rhs) : 0;
+  const int64_t xb = mp.lhs ? clamped_index(mp.lhs[j], mp.n_lhs) : j;
   const T *xr = x + (xb * M + m) * K;
   const int wpr = K / CPW, gpr = K / group;
   const uint32_t *wp = w + (e * N + n) * wpr;
@@ -186,8 +189,8 @@ __global__ __launch_bounds__(256) void qmm_plain_n_kernel(const T *__restrict__ 
   if (wi >= wpr) return;
   const int64_t j = r / M;
   const int m = (int)(r % M);
-  const int64_t e = mp.rhs ? (int64_t)mp.rhs[mp.rhs_map ? mp.rhs_map[j] : j] : 0;
-  const int64_t xb = mp.lhs ? (int64_t)mp.lhs[j] : j;
+  const int64_t e = mp.rhs ? clamped_index(mp.rhs[mp.rhs_map ? mp.rhs_map[j] : j], mp.n_rhs) : 0;
+  const int64_t xb = mp.lhs ? clamped_index(mp.lhs[j], mp.n_lhs) : j;
   const T *xr = x + (xb * M + m) * K;
   const int gpr = N / group, g = wi * CPW / group;
   const uint32_t *wp = w + e * K * wpr + wi;
@@ -235,10 +238,11 @@ static hipError_t launch_plain_t(const void *x, const uint32_t *w, const void *s
 // dt: 0 bf16, 1 fp16, 2 fp32.  rows = n_idx * M output rows (at most 2^31 - 1: they are the grid's x extent).
 hipError_t launch_qmm_plain(const void *x, const uint32_t *w, const void *scales, const void *biases,
                             const uint32_t *lhs, const uint32_t *rhs, const uint32_t *rhs_map,
-                            const uint32_t *dst_map, int64_t rows, int M, int N, int K, int group, int bits,
-                            bool transpose, int dt, void *y, hipStream_t st) {
+                            const uint32_t *dst_map, uint32_t n_lhs, uint32_t n_rhs, int64_t rows, int M, int N,
+                            int K, int group, int bits, bool transpose, int dt, void *y, hipStream_t st) {
   if (rows == 0) return hipSuccess;
-  const PlainMaps mp{lhs, rhs, rhs_map, dst_map};
+  if (transpose && (N + 3) / 4 > 65535) return hipErrorInvalidValue;  // the grid's y extent
+  const PlainMaps mp{lhs, rhs, rhs_map, dst_map, n_lhs, n_rhs};
   if (dt == 0) return launch_plain_t<uint16_t>(x, w, scales, biases, mp, rows, M, N, K, group, bits, y, transpose, st);
   if (dt == 1) return launch_plain_t<_Float16>(x, w, scales, biases, mp, rows, M, N, K, group, bits, y, transpose, st);
   return launch_plain_t<float>(x, w, scales, biases, mp, rows, M, N, K, group, bits, y, transpose, st);

@@ -181,3 +181,30 @@ def test_index_arrays_broadcast_and_batches_flatten(m):
             assert torch.allclose(y2[i, j].double(), want, rtol=1e-4, atol=1e-4), (i, j)
     with pytest.raises(m.MoeError, match="broadcast"):
         m.ops.gather_qmm(x, w_q, s, b, torch.zeros(2, dtype=torch.int32).cuda(), rhs3, True, 64, 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_indices_out_of_range_are_clamped_not_followed(m, dtype):
+    """Index values live in device memory, so the call cannot check them: an index past the last
+    matrix must read the last matrix, never memory beyond the operand.  The operands here are the
+    leading parts of larger tensors (4 of 8 weight matrices, 2 of 10 x matrices), so that an index
+    that were followed would land in memory the test owns and give a different result."""
+    torch.manual_seed(3)
+    group_size, bits, M, N, K = 64, 4, 2, 64, 128
+    w_big = (torch.randn(8, N, K) * 0.05).cuda()
+    q, s, b = m.ops.quantize(w_big.reshape(8 * N, K), group_size, bits, dtype=dtype)
+    q, s, b = q.reshape(8, N, -1), s.reshape(8, N, -1), b.reshape(8, N, -1)
+    x_big = torch.randn(10, M, K).cuda().to(dtype)
+    x, qw, sw, bw = x_big[:2], q[:4], s[:4], b[:4]  # same base pointers, fewer matrices
+    lhs = torch.tensor([0, 1, 9, 1, 0, 5], dtype=torch.int32, device="cuda")
+    rhs = torch.tensor([3, 7, 1, 4, 2, 6], dtype=torch.int32, device="cuda")
+    got = m.ops.gather_qmm(x, qw, sw, bw, lhs, rhs, True, group_size, bits)
+    want = m.ops.gather_qmm(x, qw, sw, bw, lhs.clamp(max=1), rhs.clamp(max=3), True, group_size, bits)
+    assert torch.equal(got.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       want.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    # without lhs_indices every index needs its own matrix in x
+    lib = m.capi.load_library()
+    y = torch.empty(3, M, N, dtype=torch.bfloat16, device="cuda")
+    rc = lib.mi_moe_gather_qmm(x.data_ptr(), qw.data_ptr(), sw.data_ptr(), bw.data_ptr(), None, rhs.data_ptr(), 3, 2, M, N, K,
+                               4, 1, group_size, bits, 0, y.data_ptr(), None, 0, None)
+    assert rc != 0 and b"need as many matrices in x" in lib.mi_moe_last_error()

@@ -173,6 +173,7 @@ static __device__ __align__(256) unsigned char scratch[MI_MOE_STATIC_SCRATCH_BYT
 struct mi_moe_s {
   mi_moe_config cfg;
   mi_moe_weights w;
+  int device = -1;                       // the GPU that was current in mi_moe_create: counters, streams, scratch live there
   unsigned char *scratch_dev = nullptr;  // device address of `scratch` on the handle's GPU
   uint32_t *counters = nullptr;  // device: arrival counters of the fused decode router, zero at rest
   // prefill-sized batches: the tile classes and the streamed segments are independent chains
@@ -228,7 +229,8 @@ int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_mo
   h->w = *weights;
   // the only device memory the library owns: 260 bytes of counters per handle
   const size_t cbytes = (size_t)(1 + kFusedRouterMaxTokens) * sizeof(uint32_t);
-  hipError_t e = hipMalloc(reinterpret_cast<void **>(&h->counters), cbytes);
+  hipError_t e = hipGetDevice(&h->device);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&h->counters), cbytes);
   if (e == hipSuccess) e = hipMemset(h->counters, 0, cbytes);
   // streams (default priority) and events for the independent chains of a prefill-sized forward
   for (int i = 0; i < 3 && e == hipSuccess; ++i) {
@@ -275,6 +277,10 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   if (T == 0) return 0;
   if (!x || !out) return fail("forward: x and out must be non-NULL");
   if (!aligned16(x) || !aligned16(out)) return fail("forward: x and out must be 16-byte aligned");
+  int dev = -1;
+  MI_HIP(hipGetDevice(&dev));
+  if (dev != h->device)
+    return fail("forward: the handle was created on GPU %d, the calling thread's current GPU is %d", h->device, dev);
   const mi_moe_config &c = h->cfg;
   const int64_t P = T * c.top_k;
   if (P > (int64_t)1 << 30) return fail("forward: too many (token, expert) pairs");
@@ -527,6 +533,7 @@ int mi_moe_rms_norm(const uint16_t *x, const uint16_t *weight, float eps, int64_
 int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t *out, void *workspace,
                          size_t workspace_bytes, void *stream, float *stage_ms, float *kernel_ms) try {
   if (!stage_ms) return fail("forward_timed: stage_ms is NULL");
+  for (int i = 0; i < MI_MOE_N_STAGES; ++i) stage_ms[i] = 0.f;  // what an empty batch or a failed call leaves
   hipStream_t st = static_cast<hipStream_t>(stream);
   constexpr int kEvents = MI_MOE_N_STAGES + 1 + 2 * MI_MOE_N_KERNEL_TIMES;
   hipEvent_t ev[kEvents];

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from helpers import (assert_close_bf16, bits_u16, bits_u32, bf16_tensor, device_block, errors, f32_of_bits,
-                     host_layer, host_tokens)
+                     host_layer, host_tokens, i32_tensor)
 
 pytestmark = pytest.mark.gpu
 
@@ -257,3 +257,23 @@ def test_widest_outputs_of_the_shape_sweep(orc, T, zipf):
     # the shape whose outputs are the largest of those swept (rows of 4096 values, two experts per
     # token: |out| reaches 2.7, where a bf16 ulp is 1.6e-2), under the one tolerance rule
     _run_case(orc, 4096, 8, 2, 1024, 4, T, 0, seed=200 + T, zipf_s=zipf)
+
+
+@pytest.mark.parametrize("bits,T", [(4, 1), (4, 7), (4, 40), (4, 300), (8, 1), (8, 40), (8, 300)])
+def test_one_expert_is_the_dense_quantized_mlp(orc, bits, T):
+    """n_experts = 1, top_k = 1: the router can only pick the one expert with score 1, and the block is
+    the dense quantized MLP down(silu(gate(x)) * up(x)) of mlx-lm/src/models/qwen3.rs:204-255 with
+    QuantizedLinear layers (mlx-rs/src/nn/quantized.rs:363-386).  Checked against the oracle like any
+    block, and against the chain of the op-level entry points (three quantized_matmul and a swiglu)."""
+    import mlx_rs_amd as m
+    H, I = 1024, 3072
+    got = _run_case(orc, H, 1, 1, I, bits, T, 0, seed=90 + T)
+    W = host_layer(orc, H, 1, 1, I, bits, 90 + T)
+    x = bf16_tensor(host_tokens(orc, T, H, 90 + T), "cuda")
+    mats = {n: (i32_tensor(W[n][0][0], "cuda"), bf16_tensor(W[n][1][0], "cuda"), bf16_tensor(W[n][2][0], "cuda"))
+            for n in ("gate", "up", "down")}
+    g = m.ops.quantized_matmul(x, *mats["gate"], True, 64, bits)
+    u = m.ops.quantized_matmul(x, *mats["up"], True, 64, bits)
+    h = m.ops.swiglu(g, u)
+    y = m.ops.quantized_matmul(h, *mats["down"], True, 64, bits)
+    assert_close_bf16(got, bits_u16(y), what="block vs the chain of quantized_matmul and swiglu")

@@ -21,6 +21,8 @@ def m():
     (65, 4096, 8, 2, 2, False), (17, 256, 300, 8, 0, True), (5, 128, 5, 5, 2, False),
     # 256 and more 32 x 32 logit tiles: the larger tile of the fp64 kernel (fewer: 16 x 16 tiles), ragged edges
     (2048, 256, 128, 8, 0, True), (1000, 128, 300, 4, 1, False),
+    # a single expert (the block as a dense MLP): every score is 1
+    (1, 256, 1, 1, 0, False), (40, 256, 1, 1, 2, False), (300, 256, 1, 1, 1, True),
 ])
 def test_route_bit_exact(orc, m, T, H, E, k, mode, bias):
     print(f"route T={T} H={H} E={E} k={k} mode={mode}", flush=True)
@@ -52,7 +54,8 @@ def test_route_ties_go_to_the_lower_expert(orc, m):
     assert np.array_equal(bits_u16(gs), orc.f32_to_bf16(np.full((3, k), 0.25, np.float32)))
 
 
-@pytest.mark.parametrize("P,E", [(1, 8), (8, 128), (256, 128), (4096, 8), (4097, 128), (40000, 64), (70000, 500)])
+@pytest.mark.parametrize("P,E", [(1, 8), (8, 128), (256, 128), (4096, 8), (4097, 128), (40000, 64), (70000, 500),
+                                 (1, 1), (300, 1), (5000, 1)])
 def test_dispatch_bit_exact(orc, m, P, E):
     print(f"dispatch P={P} E={E}", flush=True)
     rng = np.random.default_rng(P)

@@ -237,6 +237,8 @@ constexpr int64_t kSingleMaxP = 4096;
 // of the general path; the same outputs bit for bit.
 // LDS (dynamic, passed in): 4 * E words.  P = T * k <= kSingleMaxP.
 constexpr int kMaskTokens = 64;
+// FLAT_LOCAL: `flat` was written by this workgroup (LDS, or memory behind a barrier): plain loads.
+template <bool FLAT_LOCAL = false>
 __device__ __forceinline__ void dispatch_tokens_block(const uint32_t *flat, int T, int k, int E, uint32_t *lds,
                                       uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
                                       uint32_t *__restrict__ perm, uint32_t *__restrict__ inv_perm,
@@ -253,7 +255,7 @@ __device__ __forceinline__ void dispatch_tokens_block(const uint32_t *flat, int 
     const int j = tid + i * kDispThreads;
     es[i] = 0u;
     if (j < P) {
-      uint32_t e = load_agent(flat + j);
+      uint32_t e = FLAT_LOCAL ? flat[j] : load_agent(flat + j);
       e = e < (uint32_t)E ? e : (uint32_t)E - 1u;  // out-of-range ids are clamped, never written past LDS
       es[i] = e;
       const uint32_t t = (uint32_t)j / (uint32_t)k;

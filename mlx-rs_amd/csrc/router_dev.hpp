@@ -104,19 +104,31 @@ __device__ __forceinline__ float key_to_float(uint32_t k) {
 // The values the selection compares are exact in bf16 (rounded probabilities, or the logits
 // themselves), so value and expert id fit one 32-bit key: the upper half is the order-preserving
 // key of the bf16 value, the lower half 0xffff - expert id (lower id wins a tie).
+// a token's logits as the selecting wave holds them: lane l takes experts l, l + 64, ...
 template <int NV, bool COHERENT>
-__device__ __forceinline__ void select_wave(const uint16_t *row, int E, int k, int mode,
-                                            uint32_t *idx_out,
-                                            uint16_t *__restrict__ w_out) {
+__device__ __forceinline__ void load_logit_row(const uint16_t *row, int E, uint16_t (&bits)[NV]) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int e = j * kWave + lane;
+    bits[j] = 0;
+    if (e < E) bits[j] = COHERENT ? load_agent(row + e) : row[e];
+  }
+}
+
+// COHERENT: the selected experts are read by another workgroup of the same launch.  idx_lds (optional):
+// a second copy of the selected experts for a dispatch that follows in the same workgroup.
+template <int NV, bool COHERENT>
+__device__ __forceinline__ void select_from_bits(const uint16_t (&bits)[NV], int E, int k, int mode,
+                                                 uint32_t *idx_out, uint16_t *__restrict__ w_out,
+                                                 uint32_t *idx_lds = nullptr) {
   const int lane = lane_id();
   float g[NV], v[NV];
   float m = -INFINITY;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int e = j * kWave + lane;
-    uint16_t bits = 0;
-    if (e < E) bits = COHERENT ? load_agent(row + e) : row[e];
-    g[j] = e < E ? bf16_to_f32(bits) : -INFINITY;
+    g[j] = e < E ? bf16_to_f32(bits[j]) : -INFINITY;
     m = fmaxf(m, g[j]);
   }
   if (mode != 2) {
@@ -180,8 +192,18 @@ __device__ __forceinline__ void select_wave(const uint16_t *row, int E, int k, i
   if (lane < k) {
     if (COHERENT) store_agent(idx_out + lane, my_idx);  // read by another workgroup of this launch
     else idx_out[lane] = my_idx;
+    if (idx_lds) idx_lds[lane] = my_idx;
     w_out[lane] = f32_to_bf16(score);
   }
+}
+
+template <int NV, bool COHERENT>
+__device__ __forceinline__ void select_wave(const uint16_t *row, int E, int k, int mode,
+                                            uint32_t *idx_out,
+                                            uint16_t *__restrict__ w_out) {
+  uint16_t bits[NV];
+  load_logit_row<NV, COHERENT>(row, E, bits);
+  select_from_bits<NV, COHERENT>(bits, E, k, mode, idx_out, w_out);
 }
 
 }  // namespace mi_moe

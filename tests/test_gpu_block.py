@@ -81,11 +81,13 @@ def test_run_to_run_identical(orc):
 def test_fused_router_equals_the_separate_kernels(orc):
     """Up to 64 tokens the block runs logits + selection + dispatch as one launch; the stage-level
     entry points run them as separate kernels.  Same integers and scores, call after call (the
-    launch leaves its arrival counters at zero), across batch sizes on both sides of the switch."""
+    launch leaves its arrival counters at zero), across batch sizes on both sides of the switch, and
+    on both sides of the switch between the one-exchange kernel (up to 8 tokens) and the two-exchange
+    kernel, which share a counter."""
     import mlx_rs_amd as m
-    _fused_vs_separate(orc, m, 256, 128, 8, 128, [1, 64, 3, 64, 17, 65, 2, 40, 1])
+    _fused_vs_separate(orc, m, 256, 128, 8, 128, [1, 64, 3, 64, 17, 65, 2, 40, 1, 8, 9, 8])
     # more pairs than the dispatching workgroup has threads (60 x 20 = 1200), few experts
-    _fused_vs_separate(orc, m, 128, 32, 20, 128, [60, 33, 64])
+    _fused_vs_separate(orc, m, 128, 32, 20, 128, [60, 33, 64, 5, 60, 8])
 
 
 def _fused_vs_separate(orc, m, H, E, k, I, batches):

@@ -301,6 +301,13 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     x = f.xnorm;      // decode: written by the router kernel below
   }
 
+  // 4-bit: the tiled kernel reads activations with paired 8-blocks; h is produced that way, x is copied once
+  // per forward (prefill-sized T only): by the router's logits kernel, which holds every piece of x in
+  // registers anyway, or by a kernel of its own (light batches pair the rows beside their streamed segments)
+  const bool paired = c.bits == 4;
+  const bool streamed_first = f.tiled && !f.heavy && !ev;  // light batches start their streamed segments first
+  const bool pair_in_router = f.tiled && paired && !streamed_first && !fused_router && !plain_config(c) &&
+                              router_logits_pairs_rows(T, c.hidden);
   if (fused_router) {
     // decode: one launch for the three stages (the stage times then all land in the first)
     MI_HIP(launch_router_fused(x_in, h->w.router_w, h->w.router_bias, norm_weight, eps, f.xnorm, T, c.hidden,
@@ -312,7 +319,8 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     MI_STAGE_DONE();
     MI_STAGE_DONE();
   } else {
-    MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st));
+    MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st,
+                                pair_in_router ? f.xperm : nullptr));
     MI_STAGE_DONE();
     MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
     MI_STAGE_DONE();
@@ -332,12 +340,7 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   a.total_rows = P;
   a.max_rows_per_expert = T;  // a token picks an expert at most once
   a.max_streamed_rows = f.tiled ? f.tmr - 1 : 0;
-  // 4-bit: the tiled kernel reads activations with paired 8-blocks; h is produced that way,
-  // x is copied once per forward (prefill-sized T only)
-  const bool paired = c.bits == 4;
-  // light batches start their streamed segments first and pair the rows beside them (below)
-  const bool streamed_first = f.tiled && !f.heavy && !ev;
-  if (f.tiled && paired && !streamed_first) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
+  if (f.tiled && paired && !streamed_first && !pair_in_router) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
   // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
   a.x = x;
   a.x_perm = paired ? (f.tiled ? f.xperm : nullptr) : x;

@@ -222,8 +222,12 @@ struct GroupedArgs {
   int64_t max_streamed_rows;   // host upper bound on the longest segment that is not tiled (0: no bound known)
 };
 
+// x_paired (optional, only where router_logits_pairs_rows says so): the kernel also writes the copy of x with
+// paired 8-blocks that launch_pair_rows would make.
+bool router_logits_pairs_rows(int64_t T, int H);
 hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,
-                                int64_t T, int H, int E, uint16_t *logits, hipStream_t st);
+                                int64_t T, int H, int E, uint16_t *logits, hipStream_t st,
+                                uint16_t *x_paired = nullptr);
 hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k, int mode,
                                 uint32_t *topk_idx, uint16_t *topk_w, hipStream_t st);
 size_t dispatch_workspace_bytes(int E, int64_t P);

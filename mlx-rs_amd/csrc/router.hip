@@ -98,7 +98,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(double)))) double f64x4_t;
 template <int NT>
 __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg,
-    const float *__restrict__ bias, int64_t T, int H, int E, uint16_t *__restrict__ logits) {
+    const float *__restrict__ bias, int64_t T, int H, int E, uint16_t *__restrict__ logits,
+    uint16_t *__restrict__ x_paired) {
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, kq = lane >> 4;
@@ -135,7 +136,26 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
       R.w[a] = *reinterpret_cast<const uint4 *>(wr[a] + cc * 32);
     }
   };
-  auto multiply = [&](const Chunk &R) __attribute__((always_inline)) {
+  // x_paired (optional): a copy of x with every 8-block in the order (x0,x4,x1,x5,x2,x6,x3,x7), which the
+  // 4-bit tiled product reads.  The blocks of the first expert tile write it from the pieces they hold
+  // anyway (the four waves of a block cover every chunk of its token rows between them).
+  const bool pair_out = x_paired != nullptr && blockIdx.y == 0;  // block-uniform
+  auto multiply = [&](const Chunk &R, int cidx) __attribute__((always_inline)) {
+    if (pair_out) {
+#pragma unroll
+      for (int a = 0; a < NT; ++a) {
+        const int64_t t = t0 + 16 * a + i;
+        if (t < T) {
+          const uint4 v = R.x[a];
+          uint4 p;
+          p.x = (v.x & 0xffffu) | (v.z << 16);
+          p.y = (v.x >> 16) | (v.z & 0xffff0000u);
+          p.z = (v.y & 0xffffu) | (v.w << 16);
+          p.w = (v.y >> 16) | (v.w & 0xffff0000u);
+          *reinterpret_cast<uint4 *>(x_paired + t * H + kq * 8 + cidx * 32) = p;
+        }
+      }
+    }
     uint32_t xa[NT][4], wb[NT][4];
 #pragma unroll
     for (int a = 0; a < NT; ++a) {
@@ -163,14 +183,14 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
   for (; c + 4 < nchunks; c += 8) {  // two chunks per turn, both multiplied without a condition
     fetch(c + 4, r1);
     __builtin_amdgcn_sched_barrier(0);
-    multiply(r0);
+    multiply(r0, c);
     __builtin_amdgcn_sched_barrier(0);
     fetch(c + 8, r0);
     __builtin_amdgcn_sched_barrier(0);
-    multiply(r1);
+    multiply(r1, c + 4);
     __builtin_amdgcn_sched_barrier(0);
   }
-  if (c < nchunks) multiply(r0);  // an odd chunk left over (already fetched)
+  if (c < nchunks) multiply(r0, c);  // an odd chunk left over (already fetched)
 
   __shared__ double part[4][NT * NT][4][64];  // [wave][tile][r][lane]
 #pragma unroll
@@ -197,9 +217,12 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
   }
 }
 
+bool router_logits_pairs_rows(int64_t T, int H) { return T > 64 && H % 32 == 0; }
+
 hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,
-                                int64_t T, int H, int E, uint16_t *logits, hipStream_t st) {
+                                int64_t T, int H, int E, uint16_t *logits, hipStream_t st, uint16_t *x_paired) {
   if (T == 0) return hipSuccess;
+  if (x_paired && !router_logits_pairs_rows(T, H)) return hipErrorInvalidValue;
   if (T <= 64) {
     dim3 grid((unsigned)T, (unsigned)((E + 3) / 4));
     router_logits_kernel<1, 1><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
@@ -209,10 +232,10 @@ hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const flo
     // blocks, each a quarter of the work) when they would not (512 tokens x 128 experts: 64 tiles).
     dim3 grid((unsigned)((T + 31) / 32), (unsigned)((E + 31) / 32));
     if ((int64_t)grid.x * grid.y >= 256) {
-      router_logits_mfma_kernel<2><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+      router_logits_mfma_kernel<2><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits, x_paired);
     } else {
       grid = dim3((unsigned)((T + 15) / 16), (unsigned)((E + 15) / 16));
-      router_logits_mfma_kernel<1><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits);
+      router_logits_mfma_kernel<1><<<grid, 256, 0, st>>>(x, wg, bias, T, H, E, logits, x_paired);
     }
   }
   return hipGetLastError();

@@ -680,10 +680,11 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // wave (measured: the down product of the 128-expert layer at 80 to 256 tokens -2..-4 us; with
   // fewer rows per expert the same costs up to a microsecond: there more, smaller blocks win)
   bool pair = !GLU && two_groups && a.K <= 2048 && a.N % 32 == 0;
-  const int n_tensors = (GLU || pair) ? 4 : 2;   // scale and bias tiles per wave in LDS
+  // (the three below follow `pair`: not const, a launch that ends up with slabs gives the pairing up and sizes again)
+  int n_tensors = (GLU || pair) ? 4 : 2;   // scale and bias tiles per wave in LDS
   const int sbk = sb_range_k(a.K, kw, BITS);     // K split over the waves: tiles of a wave's range only
-  const bool zb = GLU || pair || (kw > 1 && BITS == 8);  // a block of zeros instead of a zero row (see zero_bytes)
-  const int regs_blocks = (GLU || pair) ? 4 : 6;  // blocks a CU holds by registers
+  bool zb = GLU || pair || (kw > 1 && BITS == 8);  // a block of zeros instead of a zero row (see zero_bytes)
+  int regs_blocks = (GLU || pair) ? 4 : 6;  // blocks a CU holds by registers
   // tokens staged per tile: bounded by the tile, by the longest possible segment and by LDS
   int want = TTL;
   // short segments on average: stage fewer rows where the LDS saved buys a fourth block per CU (but
@@ -717,23 +718,36 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
     const int cap = launch_blocks <= MI_MOE_CUS ? 1 : (2 * slab >= a.K ? 3 : 2);
     return b < cap ? b : cap;
   };
-  int sk = a.K;
-  int tt = fit(sk);
-  if (a.K % 512 == 0) {
-    int best_t = tt < need ? tt : need, best_b = blocks_of(sk, tt);
-    for (int cand = 4096; cand >= MI_MOE_SLAB_MIN; cand /= 2) {
-      if (cand >= a.K) continue;
-      const int t = fit(cand), tn = t < need ? t : need, b = blocks_of(cand, t);
-      if (tn > best_t || (tn == best_t && b > best_b)) {
-        sk = cand;
-        tt = t;
-        best_t = tn;
-        best_b = b;
+  int sk = a.K, tt = 0;
+  auto choose_slab = [&]() {
+    sk = a.K;
+    tt = fit(sk);
+    if (a.K % 512 == 0) {
+      int best_t = tt < need ? tt : need, best_b = blocks_of(sk, tt);
+      for (int cand = 4096; cand >= MI_MOE_SLAB_MIN; cand /= 2) {
+        if (cand >= a.K) continue;
+        const int t = fit(cand), tn = t < need ? t : need, b = blocks_of(cand, t);
+        if (tn > best_t || (tn == best_t && b > best_b)) {
+          sk = cand;
+          tt = t;
+          best_t = tn;
+          best_b = b;
+        }
       }
     }
+  };
+  choose_slab();
+  if (sk < a.K && pair) {
+    // The paired kernel stages whole rows only.  Without it the kernel keeps a zero ROW in LDS, not the 64-byte
+    // block of zeros, and two tensors' tiles per wave: the sizes are taken again for that kernel (launched with the
+    // paired kernel's sizes it would address LDS past what the launch asked for and read zeros for its scales).
+    pair = false;
+    n_tensors = 2;
+    zb = kw > 1 && BITS == 8;
+    regs_blocks = 6;
+    choose_slab();
   }
   const bool slabs = sk < a.K;
-  if (slabs) pair = false;  // (the sizes above then were on the safe side)
   size_t lds = small_lds_bytes(a.K, sk, tt, TTL, slabs ? (GLU ? 4 : 2) : n_tensors, sbk, zb);
   // with slabs a chunk's ring slot must not depend on the slab: the waves' K ranges have to start
   // at multiples of the ring depth

@@ -132,6 +132,15 @@ def test_two_token_groups_per_pass(orc, T, H, I):
     _run_case(orc, H, 8, 2, I, 4, T, 0, seed=91 + T)
 
 
+@pytest.mark.parametrize("T,H,E,k,I", [(64, 512, 64, 8, 1536), (100, 512, 64, 8, 2048), (65, 2048, 33, 6, 1536),
+                                       (160, 1024, 128, 8, 1536)])
+def test_two_token_groups_with_rows_in_slabs(orc, T, H, E, k, I):
+    # the down product of a layer with many experts (more blocks than CUs) and rows of 1536 or 2048 values at 8
+    # to 16 rows per expert: two token groups per pass, rows staged in slabs of 1024 (the last one of 512 values
+    # for 1536), one row tile per wave
+    _run_case(orc, H, E, k, I, 4, T, 0, seed=300 + T)
+
+
 @pytest.mark.parametrize("T,E,k,zipf", [(100, 16, 2, 1.5), (40, 16, 4, 1.2), (150, 32, 4, 1.0), (150, 32, 4, None)])
 def test_light_batches_tile_only_long_segments(orc, T, E, k, zipf):
     # 6 to 20 rows per expert on average (4-bit): the streamed segments lead on the caller's stream,

@@ -72,6 +72,10 @@ def test_dispatch_bit_exact(orc, m, P, E):
     (4, 32, 64, 128, 3, 2, 5),      # the reference's test shapes (K raised to a multiple of 128 for 4-bit)
     (8, 32, 64, 64, 3, 2, 1),       # ... and its exact shapes with 8-bit codes
     (4, 1, 768, 2048, 16, 40, 40), (8, 1, 256, 512, 4, 300, 300), (4, 3, 48, 256, 5, 7, 4),
+    # 4-bit plain products with two token groups per pass whose rows end up staged in slabs (more blocks than
+    # CUs, K = 1536 with a partial last slab and K = 2048): the launch gives up the paired row tiles and must
+    # size its LDS for the kernel it then runs
+    (4, 1, 512, 1536, 64, 512, 512), (4, 1, 512, 2048, 64, 768, 768), (4, 1, 1024, 2048, 40, 480, 480),
 ])
 def test_gather_qmm_matches_oracle(orc, m, bits, M, N, K, E, n_idx, xb):
     print(f"gather_qmm bits={bits} M={M} N={N} K={K} E={E} n_idx={n_idx}", flush=True)

@@ -32,9 +32,12 @@ CASES = [
     ("mixtral_8x7b", 16, None),
     ("mixtral_8x7b", 64, None),   # streamed, 16 rows per expert
     ("mixtral_8x7b", 96, None),   # 64-row tiles
+    ("mixtral_8x7b", 320, None),  # 80 rows per expert: 128-row tiles
     ("mixtral_8x7b", 2048, None),
     ("qwen3_235b_a22b", 2, None),   # K split over the waves, rows of 4096 4-bit values
     ("qwen3_235b_a22b", 32, None),  # streamed, 4-bit rows of 4096 values (two blocks per CU)
+    ("qwen3_235b_a22b", 160, None), # 10 rows per expert: two token groups per pass; the down product's rows of 1536 values in slabs of 1024 + 512
+    ("qwen3_235b_a22b", 384, 1.3),  # light batch, uneven routing
     ("qwen3_235b_a22b", 8192, 1.3),
 ]
 

@@ -82,6 +82,13 @@ def test_null_and_range_checks(lib):
     assert lib.mi_moe_gather_qmm(None, None, None, None, None, None, 2, 2, 1, 64, 64, 3, 1, 64, 5, 0,
                                  None, None, 0, None) != 0
     assert "bits" in m.capi.last_error()
+    # without lhs_indices index j reads x[j]: three indices need three matrices in x (checked before anything
+    # is launched or any pointer followed: host memory stands in for the operands here)
+    host = (C.c_char * 64)()
+    fake = C.cast(host, C.c_void_p)
+    assert lib.mi_moe_gather_qmm(fake, fake, fake, fake, None, fake, 3, 2, 1, 64, 128, 4, 1, 64, 4, 0,
+                                 fake, None, 0, None) != 0
+    assert "as many matrices in x" in m.capi.last_error()
     assert lib.mi_moe_combine(None, None, None, 4, 2, 64, None, None) != 0
     assert lib.mi_moe_swiglu(None, None, 8, None, None) != 0
     assert lib.mi_moe_stream_probe(None, 1000, None, None) != 0

@@ -234,7 +234,7 @@ def run_workload(name, args, torch, m, synth, dev):
             "gate_up_mfma_frac": gu_flops / (gu_kernel_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS if gu_kernel_ms else None,
         }
         if T == headline:
-            head = dict(ms=ms, T=T, gu_bytes=gu_bytes, dn_bytes=dn_bytes, gu_flops=gu_flops, steps=steps_done, warmup=warmup, kern=kern,
+            head = dict(stage_ms=stage, ms=ms, T=T, gu_bytes=gu_bytes, dn_bytes=dn_bytes, gu_flops=gu_flops, steps=steps_done, warmup=warmup, kern=kern,
                         class_rows=class_rows, per_row_gu_flops=2 * 2 * cfg.hidden * cfg.intermediate)
         del outs, graph
 
@@ -248,7 +248,8 @@ def run_workload(name, args, torch, m, synth, dev):
                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                     "traffic": traffic, "traffic_source": traffic_src and traffic_src + " (carried, not measured by this run)",
                     "algorithmic_bytes_per_launch": head["gu_bytes"], "kernel_us": k_ms * 1e3,
-                    "kernel_us_source": "start/end time stamps of the dispatch (hipExtLaunchKernelGGL events), mean over the timed steps",
+                    "kernel_us_source": "start/end time stamps of the dispatch (hipExtLaunchKernelGGL events), mean over the timed steps "
+                                        "(mi_moe_forward_timed: same kernels, same order and stream as mi_moe_forward at decode sizes)",
                     "stream_probe": stream_probe(m, head["gu_bytes"], dev)}
     else:
         # the dominant kernel: the tile class that holds most rows (256-row tiles at prefill sizes)
@@ -263,7 +264,12 @@ def run_workload(name, args, torch, m, synth, dev):
                     "traffic": traffic, "traffic_source": traffic_src and traffic_src + " (carried, not measured by this run)",
                     "algorithmic_flops_per_launch": k_flops, "rows_per_launch": k_rows,
                     "kernel_us": k_ms * 1e3,
-                    "kernel_us_source": "start/end time stamps of the dispatch (hipExtLaunchKernelGGL events), mean over the timed steps",
+                    "kernel_us_source": "start/end time stamps of the dispatch (hipExtLaunchKernelGGL events), mean over the timed steps, "
+                                        "kernels launched one after the other on one stream (mi_moe_forward_timed); the timed step itself "
+                                        "(ms_per_step) runs mi_moe_forward's own schedule, tile classes side by side on two to four streams",
+                    "serial_kernels_us_sum_vs_step_us": [round((sum(head["kern"]) + sum(head["stage_ms"][i] for i in (0, 1, 2, 5))) * 1e3, 1),
+                                                         round(head["ms"] * 1e3, 1)],
+                    "dense_gemm_yardstick": dense_gemm_yardstick(torch, int(round(k_rows)), 2 * cfg.intermediate, cfg.hidden, dev),
                     "gate_up_stage": {"flops": head["gu_flops"], "kernels_us": sum(head["kern"][0:4]) * 1e3,
                                       "TFLOPs": head["gu_flops"] / (sum(head["kern"][0:4]) * 1e-3) / 1e12,
                                       "frac": head["gu_flops"] / (sum(head["kern"][0:4]) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS}}
@@ -324,6 +330,30 @@ def main():
                           "ms_per_step": d["ms_per_step"], "steps": d["steps"], "config": p["config"],
                           "layer_TFLOPs": d["layer_TFLOPs"], "layer_frac_of_peak": d["layer_mfma_frac"], "detail": d}
     print(json.dumps(out))
+
+
+def dense_gemm_yardstick(torch, M, N, K, dev):
+    """A library dense bf16 GEMM of the roofline kernel's aggregate shape (M rows of the dominant tile class,
+    N = gate + up columns, K = hidden), timed the same way: what torch.matmul (hipBLASLt / rocBLAS) reaches
+    on this box for [M, K] x [K, N].  A yardstick beside the vendor peak, not on the product path: the
+    product kernel also unpacks 4-bit codes, gathers its rows and applies SwiGLU."""
+    a = torch.randn((M, K), device=dev, dtype=torch.bfloat16)
+    b = torch.randn((N, K), device=dev, dtype=torch.bfloat16)
+    out = torch.empty((M, N), device=dev, dtype=torch.bfloat16)
+    for _ in range(5):
+        torch.matmul(a, b.t(), out=out)
+    torch.cuda.synchronize()
+    reps = 30
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        torch.matmul(a, b.t(), out=out)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / reps * 1e3
+    tf = 2.0 * M * N * K / (us * 1e-6) / 1e12
+    return {"what": "torch.matmul bf16 [%d, %d] x [%d, %d]^T, yardstick only (not on the product path)" % (M, K, N, K),
+            "us": us, "TFLOPs": tf, "frac_of_peak": tf / MFMA_BF16_PEAK_TFLOPS}
 
 
 def stream_probe(m, nbytes, dev):

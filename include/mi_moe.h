@@ -26,12 +26,16 @@
  *    a time (MLX itself is not thread safe, .github/workflows/validate.yml:46), and
  *    forwards through one handle must not overlap on the GPU (use one stream per handle):
  *    a handle owns 260 bytes of device memory (arrival counters of the decode router
- *    kernel) and three streams with five events (default priority; a forward with an
- *    average of 6 rows per expert or more (17 with 8-bit weights) forks its independent
- *    kernel chains onto them from `stream` and joins them back before it returns, which is
- *    also what a graph capture of `stream` records), all
- *    created by mi_moe_create on the current device and released by mi_moe_destroy.  No
- *    other entry point allocates device memory or creates streams.
+ *    kernel), allocated by mi_moe_create on the current device and released by
+ *    mi_moe_destroy.  Each GPU has ONE set of three streams and five events (default
+ *    priority) for the whole process, created by the first mi_moe_create on that GPU and kept
+ *    until the process ends, however many handles exist: a forward with an average of 6 rows
+ *    per expert or more (17 with 8-bit weights) forks its independent kernel chains onto
+ *    them from `stream` and joins them back before it returns, which is also what a graph
+ *    capture of `stream` records (so two captures that are open at the same time on one GPU
+ *    must not both hold such a forward: a stream belongs to one capture at a time).  The
+ *    host-side fork-to-join sequence runs under a per-GPU lock.  No other entry point
+ *    allocates device memory or creates streams.
  *
  * Weight format = MLX "affine" quantisation (mlx-rs/src/ops/quantization.rs:31-47,
  * 85-87, 306-309): element c of a row lives in uint32 word c/(32/bits) at bit
@@ -239,6 +243,16 @@ int mi_moe_quantized_matmul_typed(const void *x, const uint32_t *w, const void *
                                   int32_t transpose, int32_t group_size, int32_t bits, int32_t dtype,
                                   void *y, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- a quantized linear layer with its optional bias (QuantizedLinear::forward,
+ * mlx-rs/src/nn/quantized.rs:363-386: quantized_matmul(x, w, scales, biases, transpose = true), then
+ * `+ bias` when the layer has one): y = x . dequantize(w)^T, rounded to dtype, then y + linear_bias,
+ * rounded again, as the reference's two ops.  linear_bias: [N] of element type dtype, or NULL (then this
+ * is mi_moe_quantized_matmul_typed with transpose = 1).  Same workspace. */
+int mi_moe_quantized_linear_typed(const void *x, const uint32_t *w, const void *scales,
+                                  const void *biases, const void *linear_bias, int64_t M, int32_t N,
+                                  int32_t K, int32_t group_size, int32_t bits, int32_t dtype, void *y,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- R7 silu(gate) * up on bf16 arrays (mlx_sigmoid + mlx_multiply x2,
  * mlx-rs/src/nn/activation.rs:142-144,876-880).  The block itself fuses this into
  * the gate/up product; this entry point is the stand-alone op. ---- */
@@ -269,6 +283,37 @@ int mi_moe_quantize_typed(const float *w, int64_t rows, int64_t cols, int32_t gr
 int mi_moe_dequantize_typed(const uint32_t *q, const void *scales, const void *biases, int64_t rows,
                             int64_t cols, int32_t group_size, int32_t bits, int32_t dtype,
                             float *w_hat, void *stream);
+
+/* mlx_dequantize as the reference returns it (mlx-rs/src/ops/quantization.rs:124-158): w_hat has the
+ * element type of scales and biases (dtype), [rows, cols].  The value is the fp32 one of
+ * mi_moe_dequantize_typed rounded once more to dtype. */
+int mi_moe_dequantize_native(const uint32_t *q, const void *scales, const void *biases, int64_t rows,
+                             int64_t cols, int32_t group_size, int32_t bits, int32_t dtype,
+                             void *w_hat, void *stream);
+
+/* ---- introspection; no counterpart in the reference.  The library holds one compiled variant of its
+ * two grouped-product kernels per combination of bit width, SwiGLU fusion, K split, ring depth, slab
+ * staging, token groups and tile height.  mi_moe_debug_kernel_count / _name / _launches list every variant
+ * the library contains with the number of times this process has launched it (the name stays valid
+ * until the library is unloaded): the test suite uses them to show that no variant is left
+ * without a parity-checked launch.  mi_moe_debug_plan_forward / _grouped write, into the host buffer
+ * `out` (cap bytes, NUL-terminated, entries separated by ';'), the variants with grid and LDS bytes that
+ * a forward of T tokens / one grouped product of the given extents WOULD launch, and launch nothing:
+ * they need no GPU and touch no device memory (the host-side launch rules, checked on any machine).
+ * _grouped: total_rows rows in max_active segments of at most max_rows_per_expert rows;
+ * max_streamed_rows (0 = unknown) bounds the segments that are not tiled; tile_lists non-zero = M-tile
+ * lists exist (a batch that mi_moe_forward would tile).
+ * mi_moe_debug_side_streams_created: streams the library has created in this process (three per GPU
+ * on which a handle was ever created, whatever the number of handles). ---- */
+int32_t mi_moe_debug_kernel_count(void);
+const char *mi_moe_debug_kernel_name(int32_t index);  /* NULL beyond the last variant */
+int64_t mi_moe_debug_kernel_launches(int32_t index);  /* -1 beyond the last variant */
+int mi_moe_debug_plan_forward(const mi_moe_config *cfg, int64_t T, char *out, size_t cap);
+int mi_moe_debug_plan_grouped(int32_t N, int32_t K, int32_t bits, int32_t glu, int64_t total_rows,
+                              int32_t max_active, int64_t max_rows_per_expert,
+                              int64_t max_streamed_rows, int32_t tile_lists, int32_t paired_out,
+                              char *out, size_t cap);
+int32_t mi_moe_debug_side_streams_created(void);
 
 /* ---- measurement aid; no counterpart in the reference.  A bare streaming kernel with the decode
  * grouped product's access shape (a wave reads a 16 KiB tile from each half of buf, 64 bytes per row

@@ -27,6 +27,9 @@ EXPORTS = (
     "mi_moe_quantized_matmul_workspace_size", "mi_moe_quantized_matmul", "mi_moe_swiglu", "mi_moe_combine",
     "mi_moe_quantize", "mi_moe_dequantize", "mi_moe_stream_probe",
     "mi_moe_gather_qmm_typed", "mi_moe_quantized_matmul_typed", "mi_moe_quantize_typed", "mi_moe_dequantize_typed",
+    "mi_moe_quantized_linear_typed", "mi_moe_dequantize_native",
+    "mi_moe_debug_kernel_count", "mi_moe_debug_kernel_name", "mi_moe_debug_kernel_launches", "mi_moe_debug_plan_forward", "mi_moe_debug_plan_grouped",
+    "mi_moe_debug_side_streams_created",
 )
 
 
@@ -113,13 +116,60 @@ def load_library():
         "mi_moe_quantized_matmul_typed": [vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, i32, vp, vp, sz, vp],
         "mi_moe_quantize_typed": [vp, i64, i64, i32, i32, i32, vp, vp, vp, vp],
         "mi_moe_dequantize_typed": [vp, vp, vp, i64, i64, i32, i32, i32, vp, vp],
+        "mi_moe_dequantize_native": [vp, vp, vp, i64, i64, i32, i32, i32, vp, vp],
+        "mi_moe_quantized_linear_typed": [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, vp, sz, vp],
+        "mi_moe_debug_plan_forward": [C.POINTER(Config), i64, C.c_char_p, sz],
+        "mi_moe_debug_plan_grouped": [i32, i32, i32, i32, i64, i32, i64, i64, i32, i32, C.c_char_p, sz],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = args
+    for name in ("mi_moe_debug_kernel_count", "mi_moe_debug_side_streams_created"):
+        getattr(lib, name).restype = C.c_int32
+        getattr(lib, name).argtypes = []
+    lib.mi_moe_debug_kernel_name.restype = C.c_char_p
+    lib.mi_moe_debug_kernel_name.argtypes = [i32]
+    lib.mi_moe_debug_kernel_launches.restype = i64
+    lib.mi_moe_debug_kernel_launches.argtypes = [i32]
     _lib = lib
     return lib
+
+
+def kernel_launches():
+    """{variant name: launches in this process} for every grouped-product kernel variant the library holds."""
+    lib = load_library()
+    out = {}
+    for i in range(lib.mi_moe_debug_kernel_count()):
+        out[lib.mi_moe_debug_kernel_name(i).decode()] = lib.mi_moe_debug_kernel_launches(i)
+    return out
+
+
+def _plan_entries(buf):
+    out = []
+    for item in buf.value.decode().split(";"):
+        if item:
+            name, *rest = item.split(" ")
+            out.append((name, {k: v for k, v in (r.split("=") for r in rest)}))
+    return out
+
+
+def plan_forward(cfg, tokens):
+    """The grouped-product kernel variants a forward of `tokens` tokens would launch, as
+    [(name, {"grid": "AxB", "block": "256", "lds": bytes})]; launches nothing and needs no GPU."""
+    lib = load_library()
+    buf = C.create_string_buffer(4096)
+    check(lib.mi_moe_debug_plan_forward(C.byref(cfg), tokens, buf, len(buf)))
+    return _plan_entries(buf)
+
+
+def plan_grouped(N, K, bits, glu, total_rows, max_active, max_rows_per_expert, max_streamed_rows=0, tile_lists=False,
+                 paired_out=False):
+    lib = load_library()
+    buf = C.create_string_buffer(4096)
+    check(lib.mi_moe_debug_plan_grouped(N, K, bits, int(glu), total_rows, max_active, max_rows_per_expert,
+                                        max_streamed_rows, int(tile_lists), int(paired_out), buf, len(buf)))
+    return _plan_entries(buf)
 
 
 def last_error():

@@ -2,6 +2,7 @@
 // Declarations and the reference interfaces they replace: include/mi_moe.h.
 #include "../../include/mi_moe.h"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -170,28 +171,58 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
 // kernel may use is looked up once per handle (mi_moe_create, on the handle's device) and kept there.
 static __device__ __align__(256) unsigned char scratch[MI_MOE_STATIC_SCRATCH_BYTES];
 
+// Prefill-sized batches: the tile classes and the streamed segments are independent chains (gate/up then
+// down over the same rows); three of the four run on side streams, forked from and joined back into the
+// caller's stream by events.  The streams and events belong to the GPU, not to a handle: one set per
+// device for the whole process, created by the first mi_moe_create on that device and kept until the
+// process ends (a model of 48 to 94 layers would otherwise hold 150 to 280 streams on a device with a
+// handful of hardware queues).  The host-side fork ... join sequence of a forward runs under the set's
+// lock: an event is recorded and waited for by the same forward, never by two at once.
+struct DeviceStreams {
+  std::mutex lock;
+  bool ready = false;
+  hipStream_t side[3] = {nullptr, nullptr, nullptr};
+  hipEvent_t fork = nullptr, paired = nullptr, join[3] = {nullptr, nullptr, nullptr};
+};
+constexpr int kMaxStreamDevices = 64;
+static DeviceStreams g_device_streams[kMaxStreamDevices];
+static std::atomic<int> g_side_streams_created{0};
+
+// the set of `dev` (the current device), created on first use (default priority)
+static hipError_t device_streams(int dev, DeviceStreams **out) {
+  if (dev < 0 || dev >= kMaxStreamDevices) return hipErrorInvalidDevice;
+  DeviceStreams &d = g_device_streams[dev];
+  std::lock_guard<std::mutex> g(d.lock);
+  if (!d.ready) {
+    hipError_t e = hipSuccess;
+    for (int i = 0; i < 3 && e == hipSuccess; ++i) {
+      if (!d.side[i]) {
+        e = hipStreamCreateWithFlags(&d.side[i], hipStreamNonBlocking);
+        if (e == hipSuccess) g_side_streams_created.fetch_add(1);
+      }
+      if (e == hipSuccess && !d.join[i]) e = hipEventCreateWithFlags(&d.join[i], hipEventDisableTiming);
+    }
+    if (e == hipSuccess && !d.fork) e = hipEventCreateWithFlags(&d.fork, hipEventDisableTiming);
+    if (e == hipSuccess && !d.paired) e = hipEventCreateWithFlags(&d.paired, hipEventDisableTiming);
+    if (e != hipSuccess) return e;  // what exists is kept for the next attempt
+    d.ready = true;
+  }
+  *out = &d;
+  return hipSuccess;
+}
+
 struct mi_moe_s {
   mi_moe_config cfg;
   mi_moe_weights w;
   int device = -1;                       // the GPU that was current in mi_moe_create: counters, streams, scratch live there
   unsigned char *scratch_dev = nullptr;  // device address of `scratch` on the handle's GPU
   uint32_t *counters = nullptr;  // device: arrival counters of the fused decode router, zero at rest
-  // prefill-sized batches: the tile classes and the streamed segments are independent chains
-  // (gate/up then down over the same rows); three of the four run on these streams, forked from
-  // and joined back into the caller's stream by events
-  hipStream_t side[3] = {nullptr, nullptr, nullptr};
-  hipEvent_t fork = nullptr, paired = nullptr, join[3] = {nullptr, nullptr, nullptr};
+  DeviceStreams *streams = nullptr;      // the device's side streams and events (not owned)
 };
 
 void destroy_handle(mi_moe_s *h) {
   if (!h) return;
   if (h->counters) (void)hipFree(h->counters);
-  for (int i = 0; i < 3; ++i) {
-    if (h->side[i]) (void)hipStreamDestroy(h->side[i]);
-    if (h->join[i]) (void)hipEventDestroy(h->join[i]);
-  }
-  if (h->fork) (void)hipEventDestroy(h->fork);
-  if (h->paired) (void)hipEventDestroy(h->paired);
   delete h;
 }
 
@@ -232,13 +263,8 @@ int mi_moe_create(const mi_moe_config *cfg, const mi_moe_weights *weights, mi_mo
   hipError_t e = hipGetDevice(&h->device);
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&h->counters), cbytes);
   if (e == hipSuccess) e = hipMemset(h->counters, 0, cbytes);
-  // streams (default priority) and events for the independent chains of a prefill-sized forward
-  for (int i = 0; i < 3 && e == hipSuccess; ++i) {
-    e = hipStreamCreateWithFlags(&h->side[i], hipStreamNonBlocking);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&h->join[i], hipEventDisableTiming);
-  }
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&h->fork, hipEventDisableTiming);
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&h->paired, hipEventDisableTiming);
+  // the device's streams and events for the independent chains of a prefill-sized forward
+  if (e == hipSuccess) e = device_streams(h->device, &h->streams);
   // where the built-in scratch of mi_moe_forward_static lives on this GPU
   if (e == hipSuccess) e = hipGetSymbolAddress(reinterpret_cast<void **>(&h->scratch_dev), HIP_SYMBOL(scratch));
   if (e == hipSuccess && (!h->scratch_dev || (reinterpret_cast<uintptr_t>(h->scratch_dev) & 255u))) e = hipErrorInvalidSymbol;
@@ -263,6 +289,49 @@ int mi_moe_workspace_size(const mi_moe_config *cfg, int64_t max_tokens, size_t *
   *bytes = carve_forward(*cfg, max_tokens, nullptr).bytes + 256;
   return 0;
 } MI_CATCH("workspace_size")
+
+// The operands of the two grouped products of a forward: gate/up (rows gathered from x by token, written
+// in sorted order, SwiGLU fused) and down (rows read in sorted order, written back in (token, slot) order).
+static void grouped_args(const mi_moe_config &c, const mi_moe_weights &w, const ForwardWs &f, const uint16_t *x,
+                         int64_t T, GroupedArgs &a, GroupedArgs &d) {
+  const int64_t P = T * c.top_k;
+  const bool paired = c.bits == 4;
+  a = GroupedArgs{};
+  a.work = f.work;
+  a.max_active = (int)(P < c.n_experts ? P : c.n_experts);
+  a.mtiles = f.tiled ? f.mtiles : nullptr;
+  a.max_mtiles = f.max_mtiles;
+  a.tile_cap_e = f.tiled ? c.n_experts : 0;
+  a.bits = c.bits;
+  a.total_rows = P;
+  a.max_rows_per_expert = T;  // a token picks an expert at most once
+  a.max_streamed_rows = f.tiled ? f.tmr - 1 : 0;
+  a.x = x;
+  a.x_perm = paired ? (f.tiled ? f.xperm : nullptr) : x;
+  a.x_paired = false;
+  a.y_paired = paired;
+  a.src_rows = f.src_of;
+  a.src_in_work = true;
+  a.dst_rows = nullptr;
+  a.w0 = w.gate.w; a.s0 = w.gate.scales; a.b0 = w.gate.biases;
+  a.w1 = w.up.w;   a.s1 = w.up.scales;   a.b1 = w.up.biases;
+  a.y = f.hh;
+  a.N = c.intermediate;
+  a.K = c.hidden;
+  d = a;
+  d.x = f.hh;
+  d.x_perm = f.hh;
+  d.x_paired = paired;
+  d.y_paired = false;
+  d.src_rows = nullptr;
+  d.src_in_work = false;
+  d.dst_rows = f.perm;
+  d.w0 = w.down.w; d.s0 = w.down.scales; d.b0 = w.down.biases;
+  d.w1 = nullptr; d.s1 = d.b1 = nullptr;
+  d.y = f.y;
+  d.N = c.hidden;
+  d.K = c.intermediate;
+}
 
 // The launch sequence of one forward.  ev: nullptr, or kStages + 1 events recorded on the
 // stream before the first launch and after each stage.
@@ -329,45 +398,10 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
                            f.disp_scratch, st));
     MI_STAGE_DONE();
   }
-  const int max_active = (int)(P < c.n_experts ? P : c.n_experts);
-  GroupedArgs a{};
-  a.work = f.work;
-  a.max_active = max_active;
-  a.mtiles = f.tiled ? f.mtiles : nullptr;
-  a.max_mtiles = f.max_mtiles;
-  a.tile_cap_e = f.tiled ? c.n_experts : 0;
-  a.bits = c.bits;
-  a.total_rows = P;
-  a.max_rows_per_expert = T;  // a token picks an expert at most once
-  a.max_streamed_rows = f.tiled ? f.tmr - 1 : 0;
+  GroupedArgs a{}, d{};
+  grouped_args(c, h->w, f, x, T, a, d);
+  const int max_active = a.max_active;
   if (f.tiled && paired && !streamed_first && !pair_in_router) MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, st));
-  // gate/up + SwiGLU: rows gathered from x by token, written in sorted order
-  a.x = x;
-  a.x_perm = paired ? (f.tiled ? f.xperm : nullptr) : x;
-  a.x_paired = false;
-  a.y_paired = paired;
-  a.src_rows = f.src_of;
-  a.src_in_work = true;
-  a.dst_rows = nullptr;
-  a.w0 = h->w.gate.w; a.s0 = h->w.gate.scales; a.b0 = h->w.gate.biases;
-  a.w1 = h->w.up.w;   a.s1 = h->w.up.scales;   a.b1 = h->w.up.biases;
-  a.y = f.hh;
-  a.N = c.intermediate;
-  a.K = c.hidden;
-  // down: rows read in sorted order, written back in (token, slot) order
-  GroupedArgs d = a;
-  d.x = f.hh;
-  d.x_perm = f.hh;
-  d.x_paired = paired;
-  d.y_paired = false;
-  d.src_rows = nullptr;
-  d.src_in_work = false;
-  d.dst_rows = f.perm;
-  d.w0 = h->w.down.w; d.s0 = h->w.down.scales; d.b0 = h->w.down.biases;
-  d.w1 = nullptr; d.s1 = d.b1 = nullptr;
-  d.y = f.y;
-  d.N = c.hidden;
-  d.K = c.intermediate;
   if (plain_config(c)) {
     // group sizes 32 / 128 or 2-bit codes: the plain products, one output row per sorted pair.  Row r of
     // the sorted order belongs to pair perm[r], token src_of[r], expert topk_idx[perm[r]].
@@ -394,7 +428,9 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     // join cost a few microseconds each).
     const bool exists[4] = {T > 128, T > 64, true, true};
     int n_side = 0;
-    MI_HIP(hipEventRecord(h->fork, st));
+    DeviceStreams &ds = *h->streams;
+    std::lock_guard<std::mutex> streams_guard(ds.lock);  // until the side streams have been joined back
+    MI_HIP(hipEventRecord(ds.fork, st));
     // the launches, in a function of their own: whatever happens in it, the side streams it has
     // used are joined back below (a caller must never be left with work of ours running beside
     // its stream, or with a capture that has not been joined)
@@ -404,15 +440,15 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
         MI_HIP(launch_small_qmm(d, false, st));
         for (int cls = 0; cls < 3; ++cls) {
           if (!exists[cls]) continue;
-          hipStream_t s = h->side[n_side++];
+          hipStream_t s = ds.side[n_side++];
           if (n_side == 1) {
-            MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
+            MI_HIP(hipStreamWaitEvent(s, ds.fork, 0));
             if (paired) {
               MI_HIP(launch_pair_rows(x, T, c.hidden, f.xperm, s));
-              MI_HIP(hipEventRecord(h->paired, s));
+              MI_HIP(hipEventRecord(ds.paired, s));
             }
           } else {
-            MI_HIP(hipStreamWaitEvent(s, paired ? h->paired : h->fork, 0));
+            MI_HIP(hipStreamWaitEvent(s, paired ? ds.paired : ds.fork, 0));
           }
           MI_HIP(launch_large_qmm_class(a, true, cls, s));
           MI_HIP(launch_large_qmm_class(d, false, cls, s));
@@ -430,8 +466,8 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
         // of the rows and need a stream each (one stream for them at 320 to 2048 tokens, Zipf routing: +10 to +36 %).
         const bool one_side = lead == 0;
         if (one_side) {
-          hipStream_t s = h->side[n_side++];
-          MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
+          hipStream_t s = ds.side[n_side++];
+          MI_HIP(hipStreamWaitEvent(s, ds.fork, 0));
           MI_HIP(launch_large_qmm_class(a, true, 0, st));
           MI_HIP(launch_large_qmm_class(d, false, 0, st));
           // the side stream: every gate/up launch, then every down launch (against chain after chain: -0.6 %)
@@ -446,8 +482,8 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
           if (!exists[chain]) continue;
           hipStream_t s = st;
           if (i > 0) {
-            s = h->side[n_side++];
-            MI_HIP(hipStreamWaitEvent(s, h->fork, 0));
+            s = ds.side[n_side++];
+            MI_HIP(hipStreamWaitEvent(s, ds.fork, 0));
           }
           if (chain < 3) {
             MI_HIP(launch_large_qmm_class(a, true, chain, s));
@@ -463,8 +499,8 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     const int rc = launch_chains();
     hipError_t je = hipSuccess;
     for (int i = 0; i < n_side; ++i) {
-      hipError_t e = hipEventRecord(h->join[i], h->side[i]);
-      if (e == hipSuccess) e = hipStreamWaitEvent(st, h->join[i], 0);
+      hipError_t e = hipEventRecord(ds.join[i], ds.side[i]);
+      if (e == hipSuccess) e = hipStreamWaitEvent(st, ds.join[i], 0);
       if (e != hipSuccess && je == hipSuccess) je = e;
     }
     if (rc) return rc;
@@ -840,6 +876,16 @@ int mi_moe_quantized_matmul_typed(const void *x, const uint32_t *w, const void *
                                workspace_bytes, stream);
 } MI_CATCH("quantized_matmul_typed")
 
+int mi_moe_quantized_linear_typed(const void *x, const uint32_t *w, const void *scales, const void *biases,
+                                  const void *linear_bias, int64_t M, int32_t N, int32_t K, int32_t group_size,
+                                  int32_t bits, int32_t dtype, void *y, void *workspace, size_t workspace_bytes,
+                                  void *stream) try {
+  if (quantized_matmul_impl(x, w, scales, biases, M, N, K, 1, group_size, bits, dtype, y, workspace, workspace_bytes, stream))
+    return 1;
+  if (linear_bias && M > 0) MI_HIP(launch_add_row_bias(y, linear_bias, M, N, dtype, static_cast<hipStream_t>(stream)));
+  return 0;
+} MI_CATCH("quantized_linear_typed")
+
 int mi_moe_swiglu(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out, void *stream) try {
   if (n < 0) return fail("swiglu: negative element count");
   if (n == 0) return 0;
@@ -905,13 +951,104 @@ int mi_moe_dequantize_typed(const uint32_t *q, const void *scales, const void *b
   if (check_quant_args("dequantize", rows, cols, group_size, bits) || check_dtype("dequantize", dtype)) return 1;
   if (rows * cols == 0) return 0;
   if (!q || !scales || !biases || !w_hat) return fail("dequantize: q, scales, biases and w_hat must be non-NULL");
-  MI_HIP(launch_dequantize(q, scales, biases, rows, cols, group_size, bits, w_hat, dtype, static_cast<hipStream_t>(stream)));
+  MI_HIP(launch_dequantize(q, scales, biases, rows, cols, group_size, bits, w_hat, dtype, false, static_cast<hipStream_t>(stream)));
   return 0;
 } MI_CATCH("dequantize_typed")
+
+int mi_moe_dequantize_native(const uint32_t *q, const void *scales, const void *biases, int64_t rows,
+                             int64_t cols, int32_t group_size, int32_t bits, int32_t dtype, void *w_hat,
+                             void *stream) try {
+  if (check_quant_args("dequantize", rows, cols, group_size, bits) || check_dtype("dequantize", dtype)) return 1;
+  if (rows * cols == 0) return 0;
+  if (!q || !scales || !biases || !w_hat) return fail("dequantize: q, scales, biases and w_hat must be non-NULL");
+  MI_HIP(launch_dequantize(q, scales, biases, rows, cols, group_size, bits, w_hat, dtype, true, static_cast<hipStream_t>(stream)));
+  return 0;
+} MI_CATCH("dequantize_native")
 
 int mi_moe_dequantize(const uint32_t *q, const uint16_t *scales, const uint16_t *biases, int64_t rows,
                       int64_t cols, int32_t group_size, int32_t bits, float *w_hat, void *stream) try {
   return mi_moe_dequantize_typed(q, scales, biases, rows, cols, group_size, bits, MI_MOE_DTYPE_BF16, w_hat, stream);
 } MI_CATCH("dequantize")
+
+// ------------------------------------------------------------------ introspection (no counterpart in the reference)
+
+int32_t mi_moe_debug_kernel_count(void) {
+  int32_t n = 0;
+  for (const KernelSlot *s = kernel_slots(); s; s = s->next) ++n;
+  return n;
+}
+
+const char *mi_moe_debug_kernel_name(int32_t index) {
+  int32_t i = 0;
+  for (KernelSlot *s = kernel_slots(); s; s = s->next, ++i)
+    if (i == index) return s->name;
+  return nullptr;
+}
+
+int64_t mi_moe_debug_kernel_launches(int32_t index) {
+  int32_t i = 0;
+  for (KernelSlot *s = kernel_slots(); s; s = s->next, ++i)
+    if (i == index) return (int64_t)__atomic_load_n(&s->launches, __ATOMIC_RELAXED);
+  return -1;
+}
+
+namespace {
+// nothing is launched while one of these lives on the calling thread: launch_kernel writes to `plan` instead
+struct PlanScope {
+  LaunchPlan plan;
+  PlanScope(char *out, size_t cap) : plan{out, cap} {
+    if (out && cap) out[0] = 0;
+    g_launch_plan = &plan;
+  }
+  ~PlanScope() { g_launch_plan = nullptr; }
+};
+}  // namespace
+
+int mi_moe_debug_plan_grouped(int32_t N, int32_t K, int32_t bits, int32_t glu, int64_t total_rows, int32_t max_active,
+                              int64_t max_rows_per_expert, int64_t max_streamed_rows, int32_t tile_lists,
+                              int32_t paired_out, char *out, size_t cap) try {
+  if (bits != 4 && bits != 8) return fail("debug_plan_grouped: the tuned kernels take 4- or 8-bit codes, got %d", bits);
+  if (N <= 0 || K <= 0 || K % 64 || (bits == 4 && K % 128) || N % 16)
+    return fail("debug_plan_grouped: N must be a multiple of 16, K of 64 (4-bit: 128), got %d, %d", N, K);
+  if (total_rows < 0 || max_active < 0 || max_rows_per_expert < 0 || max_streamed_rows < 0) return fail("debug_plan_grouped: negative count");
+  static const uint32_t dummy[4] = {0, 0, 0, 0};  // never read: nothing is launched
+  GroupedArgs a{};
+  a.x = a.x_perm = reinterpret_cast<const uint16_t *>(dummy);
+  a.work = dummy;
+  a.w0 = a.w1 = dummy;
+  a.N = N; a.K = K; a.bits = bits;
+  a.total_rows = total_rows;
+  a.max_active = max_active;
+  a.max_rows_per_expert = max_rows_per_expert;
+  a.max_streamed_rows = max_streamed_rows;
+  a.y_paired = paired_out != 0;
+  if (tile_lists) {
+    a.mtiles = dummy;
+    a.max_mtiles = (int)(total_rows / kBigTileM + max_active);
+    a.tile_cap_e = max_active;
+  }
+  PlanScope scope(out, cap);
+  MI_HIP(launch_grouped_qmm(a, glu != 0, nullptr));
+  return 0;
+} MI_CATCH("debug_plan_grouped")
+
+int mi_moe_debug_plan_forward(const mi_moe_config *cfg, int64_t T, char *out, size_t cap) try {
+  if (check_config(cfg)) return 1;
+  if (T < 1 || T * cfg->top_k > (int64_t)1 << 30) return fail("debug_plan_forward: token count out of range");
+  if (plain_config(*cfg)) {
+    if (out && cap) out[0] = 0;
+    return 0;  // the plain products: none of the listed kernels
+  }
+  const ForwardWs f = carve_forward(*cfg, T, reinterpret_cast<void *>(uintptr_t{256}));
+  mi_moe_weights w{};
+  GroupedArgs a{}, d{};
+  grouped_args(*cfg, w, f, reinterpret_cast<const uint16_t *>(uintptr_t{256}), T, a, d);
+  PlanScope scope(out, cap);
+  MI_HIP(launch_grouped_qmm(a, true, nullptr));
+  MI_HIP(launch_grouped_qmm(d, false, nullptr));
+  return 0;
+} MI_CATCH("debug_plan_forward")
+
+int32_t mi_moe_debug_side_streams_created(void) { return g_side_streams_created.load(); }
 
 }  // extern "C"

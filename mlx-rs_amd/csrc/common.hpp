@@ -187,8 +187,36 @@ struct KernelTimer {
   bool used = false;  // a kernel was launched with these events
 };
 extern thread_local KernelTimer *g_kernel_timer;
+
+// ---------------------------------------------------------------- which kernels the library holds, and which ran
+// Every instantiation of a grouped-product kernel that a launcher can reach owns one slot (a static of
+// the launcher's template, registered when the library is loaded), so the list is complete whether or
+// not a kernel has ever run.  launch_kernel counts the launch in the slot.  With a plan installed on the
+// calling thread (mi_moe_debug_plan) nothing is launched: the slot's name, grid and LDS size are
+// written to the plan instead, which lets the launchers' host-side choices be checked without a GPU.
+struct KernelSlot {
+  char name[96];
+  unsigned long long launches = 0;  // updated with __atomic builtins
+  KernelSlot *next = nullptr;
+  KernelSlot(const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+};
+KernelSlot *kernel_slots();  // head of the list
+struct LaunchPlan {
+  char *out;
+  size_t cap, len = 0;
+  int n = 0;
+};
+extern thread_local LaunchPlan *g_launch_plan;
+void plan_note(const KernelSlot &slot, dim3 grid, dim3 block, size_t lds);
+inline bool planning() { return g_launch_plan != nullptr; }
+
 template <class Kernel, class... Args>
-inline void launch_kernel(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t st, Args... args) {
+inline void launch_kernel(KernelSlot &slot, Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t st, Args... args) {
+  if (planning()) {
+    plan_note(slot, grid, block, lds);
+    return;
+  }
+  __atomic_fetch_add(&slot.launches, 1ull, __ATOMIC_RELAXED);
   if (KernelTimer *t = g_kernel_timer) {
     hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)lds, st, t->start, t->stop, 0, args...);
     t->used = true;
@@ -278,7 +306,8 @@ hipError_t launch_qmm_plain(const void *x, const uint32_t *w, const void *scales
 hipError_t launch_quantize(const float *w, int64_t rows, int64_t cols, int group, int bits,
                            uint32_t *q, void *s, void *b, int dt, hipStream_t st);
 hipError_t launch_dequantize(const uint32_t *q, const void *s, const void *b,
-                             int64_t rows, int64_t cols, int group, int bits, float *out, int dt,
+                             int64_t rows, int64_t cols, int group, int bits, void *out, int dt, bool native_out,
                              hipStream_t st);
+hipError_t launch_add_row_bias(void *y, const void *bias, int64_t M, int N, int dt, hipStream_t st);
 
 }  // namespace mi_moe

@@ -11,6 +11,8 @@
 // group, in fp32.  The integer codes are exact in bf16, so the matrix cores multiply raw
 // codes (no per-element dequantisation, no rounding of w_hat), and scale and bias are
 // applied once per group to the fp32 partial sums.
+#include <cstdarg>
+#include <cstdio>
 #include <cstdlib>
 
 #include "common.hpp"
@@ -18,6 +20,30 @@
 namespace mi_moe {
 
 thread_local KernelTimer *g_kernel_timer = nullptr;
+thread_local LaunchPlan *g_launch_plan = nullptr;
+
+// the list of kernel slots: its head is constant-initialised, so slots may register in any order
+// while the library's static objects are constructed
+static KernelSlot *g_slot_head = nullptr;
+KernelSlot *kernel_slots() { return g_slot_head; }
+KernelSlot::KernelSlot(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(name, sizeof name, fmt, ap);
+  va_end(ap);
+  next = g_slot_head;
+  g_slot_head = this;
+}
+void plan_note(const KernelSlot &slot, dim3 grid, dim3 block, size_t lds) {
+  LaunchPlan *p = g_launch_plan;
+  if (!p) return;
+  ++p->n;
+  if (p->out && p->len < p->cap) {
+    const int w = snprintf(p->out + p->len, p->cap - p->len, "%s%s grid=%ux%u block=%u lds=%zu", p->len ? ";" : "", slot.name,
+                           grid.x, grid.y, block.x, lds);
+    if (w > 0) p->len = p->len + (size_t)w < p->cap ? p->len + (size_t)w : p->cap - 1;
+  }
+}
 
 __device__ __forceinline__ f32x4_t mfma16(const uint32_t (&a)[4], const uint32_t (&b)[4],
                                           f32x4_t c) {
@@ -142,6 +168,30 @@ __host__ __device__ constexpr size_t small_lds_bytes(int K, int sk, int tt, int 
          (size_t)4 * n_tensors * sb_tile_bytes(sbk > 0 && sk == K ? sbk : sb_tile_k(K, sk));
 }
 
+// The LDS layout of one instantiation, in one place: the kernel takes its offsets from here and the
+// launcher asks for lds_bytes() of the very instantiation it launches, with the values it passes.
+template <int BITS, bool GLU, int KW, bool SLABS, int TG, bool PAIR>
+struct SmallLayout {
+  static constexpr bool TWO = GLU || PAIR;                   // two weight tiles per chunk
+  static constexpr bool ZB = TWO || (KW > 1 && BITS == 8);   // 64 bytes of zeros, not a zero row (zero_bytes)
+  static constexpr int TT = BITS == 4 ? 8 : 16;              // token slots of one MFMA tile
+  static constexpr int TTL = TT * TG;                        // token slots of one pass
+  static constexpr int NTEN = TWO ? 4 : 2;                   // scale and bias tiles per wave
+  // sk: K values of a token row staged at a time (K itself without slabs)
+  // K values of a weight row whose scales (biases) a wave parks: its own K range, the slab, or the row
+  __host__ __device__ static constexpr int sb_k(int K, int sk) {
+    const int rk = SLABS ? 0 : sb_range_k(K, KW, BITS);
+    return KW > 1 && rk > 0 ? rk : sb_tile_k(K, SLABS ? sk : K);
+  }
+  __host__ __device__ static constexpr size_t gs_offset(int sk, int tt) { return (size_t)tt * x_stride_bytes(sk) + zero_bytes(sk, ZB); }
+  __host__ __device__ static constexpr size_t sb_offset(int sk, int tt) { return gs_offset(sk, tt) + (size_t)(sk / 64) * TTL * 4; }
+  __host__ __device__ static constexpr size_t lds_bytes(int K, int sk, int tt) {
+    return sb_offset(sk, tt) + (size_t)4 * NTEN * sb_tile_bytes(sb_k(K, sk));
+  }
+  // statically allocated beside it: the partial sums of a K split
+  static constexpr size_t static_bytes = KW > 1 ? (size_t)KW * (4 / KW) * (TWO ? 2 : 1) * 4 * 64 * 4 + 16 : 16;
+};
+
 // PRECISE: the ring's refills are issued without a condition (chunk index clamped), so the compiler
 // waits for exactly the chunk it needs and a wave really keeps D chunks in flight.  With the
 // conditional refills it waits for every load in flight before each chunk; that is the faster form
@@ -162,11 +212,12 @@ template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG, int D, b
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D > MI_MOE_RING ? 2 : 3, 8)))
 void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   static_assert(!PAIR || (!GLU && KW == 1 && !SLABS), "two row tiles per wave: plain product, whole rows, K not split");
-  constexpr bool TWO = GLU || PAIR;  // two weight tiles per chunk
+  using L = SmallLayout<BITS, GLU, KW, SLABS, TG, PAIR>;
+  constexpr bool TWO = L::TWO;  // two weight tiles per chunk
   // lanes without a token read a 64-byte block of zeros (see zero_bytes); with 4-bit codes and K split over
   // the waves (a few tokens of a 128-expert layer) the plain kernel keeps its zero row: the block costs it
   // registers and a quarter of a microsecond there
-  constexpr bool ZB = TWO || (KW > 1 && BITS == 8);
+  constexpr bool ZB = L::ZB;
   static_assert(TG == 1 || (TG == 2 && BITS == 4 && KW == 1), "two token groups: 4-bit, K not split over waves");
   constexpr int NW = 4 / KW;                    // row tiles per block
   constexpr int CH = BITS == 4 ? 128 : 64;      // codes per chunk (one 16-byte load per lane)
@@ -225,7 +276,7 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
   const int sb_rk = SLABS ? 0 : sb_range_k(K, KW, BITS);  // K split over the waves: the tiles of the wave's range
   const bool sb_range = KW > 1 && sb_rk > 0;
   const bool sb_whole = !sb_range && (!SLABS || sb_tile_k(K, sk) == K);  // scale / bias tiles of the whole row
-  const int sbt = sb_tile_bytes(sb_range ? sb_rk : sb_tile_k(K, sk));  // bytes of one tensor's scale (bias) tile in LDS
+  const int sbt = sb_tile_bytes(L::sb_k(K, sk));  // bytes of one tensor's scale (bias) tile in LDS
   const int sb_groups = sb_range ? sb_rk / 64 : (sb_whole ? groups_per_row : groups_per_slab);  // per row in LDS
 
   // issue every global load of chunk ch into R
@@ -268,7 +319,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
   // scales and biases of the wave's 16 rows: K/2 contiguous bytes per tensor, fetched with
   // fully coalesced 16-byte loads now and parked in LDS (wave-private) before the chunk loop
-  constexpr int NTEN = 2 * NM;  // tensors: scales, biases (x gate, up)
+  constexpr int NTEN = L::NTEN;  // tensors: scales, biases (x gate, up)
+  static_assert(NTEN == 2 * NM, "tiles per wave");
   constexpr int SBI = KW > 1 && BITS == 8 ? 4 : 2;  // 16-byte loads per lane per tensor kept in registers
   const uint32_t sb_goff = (uint32_t)n0 * groups_per_row * 2 + lane * 16;
   u32x4_t sbv[NTEN][SBI];
@@ -299,8 +351,8 @@ void qmm_small_kernel(GroupedArgs a, int tt, int sk_arg) {
 
   extern __shared__ __align__(16) unsigned char lds[];
   unsigned char *lds_x = lds;
-  float *lds_gs = reinterpret_cast<float *>(lds + tt * xstride + zero_bytes(sk, ZB));  // [groups of the slab][TTL] sums of x
-  unsigned char *lds_sb = lds + tt * xstride + zero_bytes(sk, ZB) + groups_per_slab * TTL * 4 + wave * NTEN * sbt;
+  float *lds_gs = reinterpret_cast<float *>(lds + L::gs_offset(sk, tt));  // [groups of the slab][TTL] sums of x
+  unsigned char *lds_sb = lds + L::sb_offset(sk, tt) + wave * NTEN * sbt;
 
   // park the scale / bias tiles (wave-private: no barrier needed, only the wave's own wait);
   // long rows in slabs: each slab brings its own piece (see the slab loop)
@@ -659,8 +711,31 @@ static bool allow_lds(const void *fn, size_t lds) {
   return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess;
 }
 
+// what launch_small has chosen, handed to the one instantiation that runs it
+struct LaunchChoice {
+  const GroupedArgs *a;
+  dim3 grid;
+  size_t lds;  // the size the choice was made with
+  int tt, sk;
+  hipStream_t st;
+};
+template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG, int D, bool PAIR>
+KernelSlot small_slot("qmm_small_kernel<%d,%d,%d,%d,%d,%d,%d,%d>", BITS, (int)GLU, KW, (int)PRECISE, (int)SLABS, TG, D, (int)PAIR);
+
+template <int BITS, bool GLU, int KW, bool PRECISE, bool SLABS, int TG, int D, bool PAIR>
+static hipError_t launch_small_as(const LaunchChoice &c) {
+  using L = SmallLayout<BITS, GLU, KW, SLABS, TG, PAIR>;
+  const GroupedArgs &a = *c.a;
+  const size_t need = L::lds_bytes(a.K, SLABS ? c.sk : a.K, c.tt);
+  if (need != c.lds || need + L::static_bytes > (size_t)160 * 1024 || c.tt < 1 || (!SLABS && c.sk != a.K)) return hipErrorInvalidConfiguration;
+  const auto kernel = &qmm_small_kernel<BITS, GLU, KW, PRECISE, SLABS, TG, D, PAIR>;
+  if (!planning() && !allow_lds(reinterpret_cast<const void *>(kernel), need)) return hipGetLastError();
+  launch_kernel(small_slot<BITS, GLU, KW, PRECISE, SLABS, TG, D, PAIR>, kernel, c.grid, dim3(256), need, c.st, a, c.tt, c.sk);
+  return planning() ? hipSuccess : hipGetLastError();
+}
+
 template <int BITS, bool GLU>
-static void launch_small(const GroupedArgs &a, hipStream_t st) {
+static hipError_t launch_small(const GroupedArgs &a, hipStream_t st) {
   constexpr int TT = BITS == 4 ? 8 : 16;  // token slots of one MFMA tile
   // split K over the 4 waves of a block when there are too few row tiles to fill the chip
   const int64_t tiles = (int64_t)(a.N / 16) * a.max_active;
@@ -759,7 +834,10 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   const int64_t grid_blocks = (int64_t)((a.N + 16 * (4 / kw) - 1) / (16 * (4 / kw))) * a.max_active;
   const bool deeper = deep && (by_lds0 <= 1 || grid_blocks <= MI_MOE_CUS) && !slabs &&
                       ((chunks + kw - 1) / kw) % (2 * MI_MOE_RING_DEEP) == 0;
-  if (sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % (deep ? MI_MOE_RING_DEEP : MI_MOE_RING) != 0) {
+  // K goes unsplit after all when slabs and the split do not line up, or when the split's extra LDS (the
+  // partial sums of the waves, up to 8 KB) is what does not fit beside rows this long
+  const bool split_misfit = kw > 1 && lds + 4096 * (GLU ? 2 : 1) + 16 > (size_t)160 * 1024;
+  if ((sk < a.K && kw > 1 && ((chunks + kw - 1) / kw) % (deep ? MI_MOE_RING_DEEP : MI_MOE_RING) != 0) || split_misfit) {
     kw = 1;  // (and with it the zero row instead of the block of zeros)
     lds = small_lds_bytes(a.K, sk, tt, TTL, GLU ? 4 : 2, 0, GLU);
   }
@@ -769,45 +847,46 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   // blocks a CU holds: by LDS (160 KB) and by registers (4 with the gate/up kernel, 6 otherwise)
   const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
   const bool precise = (by_lds < regs_blocks ? by_lds : regs_blocks) <= MI_MOE_PRECISE_BELOW;
-#define MI_SMALL_LAUNCH(KWV, PR, SL, TGV, DV)                                                    \
-  do {                                                                                         \
-    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV>), lds)) return; \
-    launch_kernel(qmm_small_kernel<BITS, GLU, KWV, PR, SL, TGV, DV>, grid, dim3(256), lds, st, a, tt, sk); \
+  // The launch asks for the LDS of the very instantiation it starts, from that instantiation's own layout and
+  // the values the kernel is given; the size the search above worked with must be that size (a launch
+  // whose two sides disagree is refused: it would address LDS it did not ask for).
+  const LaunchChoice ch{&a, grid, lds, tt, sk, st};
+  hipError_t err = hipSuccess;
+#define MI_SMALL_LAUNCH(KWV, PR, SL, TGV, DV, PAIRV) err = launch_small_as<BITS, GLU, KWV, PR, SL, TGV, DV, PAIRV>(ch)
+  // Ring depth: only 8-bit codes go deeper than MI_MOE_RING (`deep`, `deeper` are false with 4-bit codes).  With
+  // 8-bit codes and whole rows the unconditional ring is always a deep one (what makes it unconditional, two
+  // blocks per CU or fewer, is what makes it deep); the gate/up kernel with K unsplit has no use for sixteen chunks
+  // (one block per CU means rows that long are in slabs, a launch of at most one block per CU has K split).
+#define MI_SMALL(KWV, TGV)                                                                      \
+  do {                                                                                          \
+    if constexpr (BITS == 8) {                                                                  \
+      if (slabs && deep) { MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING_DEEP, false); break; }              \
+      if (slabs) { MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING, false); break; }          \
+      if (precise) {                                                                            \
+        if constexpr (!(GLU && KWV == 1)) {                                                     \
+          if (deeper) { MI_SMALL_LAUNCH(KWV, true, false, TGV, 2 * MI_MOE_RING_DEEP, false); break; } \
+        }                                                                                       \
+        MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING_DEEP, false);                        \
+        break;                                                                                  \
+      }                                                                                         \
+      MI_SMALL_LAUNCH(KWV, false, false, TGV, MI_MOE_RING, false);                              \
+    } else {                                                                                    \
+      if (slabs) MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING, false); /* long rows: few blocks per CU anyway */ \
+      else if (precise) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING, false);             \
+      else MI_SMALL_LAUNCH(KWV, false, false, TGV, MI_MOE_RING, false);                         \
+    }                                                                                           \
   } while (0)
-#define MI_SMALL(KWV, TGV)                                                                     \
-  do {                                                                                         \
-    if (slabs && deep) MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING_DEEP);                \
-    else if (slabs) MI_SMALL_LAUNCH(KWV, true, true, TGV, MI_MOE_RING); /* long rows: few blocks per CU anyway */ \
-    else if (precise && deeper) MI_SMALL_LAUNCH(KWV, true, false, TGV, 2 * MI_MOE_RING_DEEP);  \
-    else if (precise && deep) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING_DEEP);        \
-    else if (precise) MI_SMALL_LAUNCH(KWV, true, false, TGV, MI_MOE_RING);                     \
-    else MI_SMALL_LAUNCH(KWV, false, false, TGV, MI_MOE_RING);                                 \
-  } while (0)
-  if constexpr (!GLU) {
-    if (pair) {  // (kw = 1, whole rows)
-#define MI_PAIR_LAUNCH(PR, TGV, DV)                                                              \
-  do {                                                                                         \
-    if (!allow_lds(reinterpret_cast<const void *>(&qmm_small_kernel<BITS, false, 1, PR, false, TGV, DV, true>), lds)) return; \
-    launch_kernel(qmm_small_kernel<BITS, false, 1, PR, false, TGV, DV, true>, grid, dim3(256), lds, st, a, tt, sk); \
-  } while (0)
-      if constexpr (BITS == 4) {
-        if (two_groups) {
-          if (precise) MI_PAIR_LAUNCH(true, 2, MI_MOE_RING);
-          else MI_PAIR_LAUNCH(false, 2, MI_MOE_RING);
-          return;
-        }
-      }
-      if (precise && deep) MI_PAIR_LAUNCH(true, 1, MI_MOE_RING_DEEP);
-      else if (precise) MI_PAIR_LAUNCH(true, 1, MI_MOE_RING);
-      else MI_PAIR_LAUNCH(false, 1, MI_MOE_RING);
-#undef MI_PAIR_LAUNCH
-      return;
+  if constexpr (!GLU && BITS == 4) {
+    if (pair) {  // (two token groups, kw = 1, whole rows)
+      if (precise) MI_SMALL_LAUNCH(1, true, false, 2, MI_MOE_RING, true);
+      else MI_SMALL_LAUNCH(1, false, false, 2, MI_MOE_RING, true);
+      return err;
     }
   }
   if constexpr (BITS == 4) {
     if (two_groups) {
       MI_SMALL(1, 2);
-      return;
+      return err;
     }
   }
   if (kw == 4) MI_SMALL(4, 1);
@@ -815,19 +894,14 @@ static void launch_small(const GroupedArgs &a, hipStream_t st) {
   else MI_SMALL(1, 1);
 #undef MI_SMALL_LAUNCH
 #undef MI_SMALL
+  return err;
 }
 
 // the streaming kernel on its own: segments the dispatch did not list as M tiles
 hipError_t launch_small_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {
   if (a.max_active <= 0 || a.total_rows <= 0) return hipSuccess;
-  if (a.bits == 4) {
-    if (glu) launch_small<4, true>(a, st);
-    else launch_small<4, false>(a, st);
-  } else {
-    if (glu) launch_small<8, true>(a, st);
-    else launch_small<8, false>(a, st);
-  }
-  return hipGetLastError();
+  if (a.bits == 4) return glu ? launch_small<4, true>(a, st) : launch_small<4, false>(a, st);
+  return glu ? launch_small<8, true>(a, st) : launch_small<8, false>(a, st);
 }
 
 hipError_t launch_grouped_qmm(const GroupedArgs &a, bool glu, hipStream_t st) {

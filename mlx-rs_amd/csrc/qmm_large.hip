@@ -405,6 +405,9 @@ hipError_t launch_pair_rows(const uint16_t *x, int64_t rows, int K, uint16_t *ou
 }
 
 template <int BITS, bool GLU, int MT>
+KernelSlot large_slot("qmm_large_kernel<%d,%d,%d>", BITS, (int)GLU, MT);
+
+template <int BITS, bool GLU, int MT>
 static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int list_cap, int sub_log2, hipStream_t st) {
   const int cap = list_cap << sub_log2;  // M tiles of this kernel's size
   const int ni = GLU ? 128 : 256;
@@ -422,17 +425,18 @@ static hipError_t launch_one(const GroupedArgs &a, const uint32_t *tiles, int li
   constexpr int kMaxDevices = 64;
   static std::atomic<bool> raised[kMaxDevices];
   int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-  if (dev < 0 || dev >= kMaxDevices || !raised[dev].load(std::memory_order_acquire)) {
+  if (!planning())
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (!planning() && (dev < 0 || dev >= kMaxDevices || !raised[dev].load(std::memory_order_acquire))) {
     if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_large_kernel<BITS, GLU, MT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         e != hipSuccess)
       return e;
     if (dev >= 0 && dev < kMaxDevices) raised[dev].store(true, std::memory_order_release);
   }
-  launch_kernel(qmm_large_kernel<BITS, GLU, MT>, dim3(grid), dim3(NTHREADS), lds, st, a, tiles, n_ntiles, list_cap, chunk,
-                sub_log2);
-  return hipGetLastError();
+  launch_kernel(large_slot<BITS, GLU, MT>, qmm_large_kernel<BITS, GLU, MT>, dim3(grid), dim3(NTHREADS), lds, st, a, tiles,
+                n_ntiles, list_cap, chunk, sub_log2);
+  return planning() ? hipSuccess : hipGetLastError();
 }
 
 // class 0 / 1 / 2 = the 256- / 128- / 64-row tile list.  A segment is at most max_rows_per_expert

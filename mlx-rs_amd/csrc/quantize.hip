@@ -76,12 +76,13 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__
   }
 }
 
-template <class T>
+// O: element type of the result (float, or the type of scales and biases: what mlx_dequantize returns)
+template <class T, class O>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t *__restrict__ q,
                                                          const T *__restrict__ scales,
                                                          const T *__restrict__ biases,
                                                          int64_t n_words, int group, int bits,
-                                                         float *__restrict__ out) {
+                                                         O *__restrict__ out) {
 #pragma clang fp contract(off)
   const int per_word = 32 / bits;
   const int64_t wi = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t *__restr
   uint32_t word = q[wi];
   const uint32_t m = (1u << bits) - 1u;
   for (int j = 0; j < per_word; ++j) {
-    out[wi * per_word + j] = s * (float)(word & m) + b;  // two roundings (contraction is off)
+    Elem<O>::store(out + wi * per_word + j, s * (float)(word & m) + b);  // two fp32 roundings (contraction is off), then O's
     word >>= bits;
   }
 }
@@ -108,15 +109,37 @@ hipError_t launch_quantize(const float *w, int64_t rows, int64_t cols, int group
   return hipGetLastError();
 }
 
+// native_out: the result has the element type of scales and biases (dt); otherwise float
 hipError_t launch_dequantize(const uint32_t *q, const void *s, const void *b,
-                             int64_t rows, int64_t cols, int group, int bits, float *out, int dt,
+                             int64_t rows, int64_t cols, int group, int bits, void *out, int dt, bool native_out,
                              hipStream_t st) {
   const int64_t n_words = rows * cols * bits / 32;
   if (n_words == 0) return hipSuccess;
   const unsigned grid = (unsigned)((n_words + 255) / 256);
-  if (dt == 0) dequantize_kernel<uint16_t><<<grid, 256, 0, st>>>(q, (const uint16_t *)s, (const uint16_t *)b, n_words, group, bits, out);
-  else if (dt == 1) dequantize_kernel<_Float16><<<grid, 256, 0, st>>>(q, (const _Float16 *)s, (const _Float16 *)b, n_words, group, bits, out);
-  else dequantize_kernel<float><<<grid, 256, 0, st>>>(q, (const float *)s, (const float *)b, n_words, group, bits, out);
+  if (dt == 0 && native_out) dequantize_kernel<uint16_t, uint16_t><<<grid, 256, 0, st>>>(q, (const uint16_t *)s, (const uint16_t *)b, n_words, group, bits, (uint16_t *)out);
+  else if (dt == 0) dequantize_kernel<uint16_t, float><<<grid, 256, 0, st>>>(q, (const uint16_t *)s, (const uint16_t *)b, n_words, group, bits, (float *)out);
+  else if (dt == 1 && native_out) dequantize_kernel<_Float16, _Float16><<<grid, 256, 0, st>>>(q, (const _Float16 *)s, (const _Float16 *)b, n_words, group, bits, (_Float16 *)out);
+  else if (dt == 1) dequantize_kernel<_Float16, float><<<grid, 256, 0, st>>>(q, (const _Float16 *)s, (const _Float16 *)b, n_words, group, bits, (float *)out);
+  else dequantize_kernel<float, float><<<grid, 256, 0, st>>>(q, (const float *)s, (const float *)b, n_words, group, bits, (float *)out);
+  return hipGetLastError();
+}
+
+// y[m][n] += bias[n], one rounding to T: the add that follows the product in a linear layer with a bias
+// (mlx-rs/src/nn/quantized.rs:363-386: quantized_matmul, then add, each rounded to the element type)
+template <class T>
+__global__ __launch_bounds__(256) void add_row_bias_kernel(T *__restrict__ y, const T *__restrict__ bias, int64_t n, int N) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  Elem<T>::store(y + i, Elem<T>::load(y + i) + Elem<T>::load(bias + i % N));
+}
+
+hipError_t launch_add_row_bias(void *y, const void *bias, int64_t M, int N, int dt, hipStream_t st) {
+  const int64_t n = M * N;
+  if (n == 0) return hipSuccess;
+  const unsigned grid = (unsigned)((n + 255) / 256);
+  if (dt == 0) add_row_bias_kernel<uint16_t><<<grid, 256, 0, st>>>((uint16_t *)y, (const uint16_t *)bias, n, N);
+  else if (dt == 1) add_row_bias_kernel<_Float16><<<grid, 256, 0, st>>>((_Float16 *)y, (const _Float16 *)bias, n, N);
+  else add_row_bias_kernel<float><<<grid, 256, 0, st>>>((float *)y, (const float *)bias, n, N);
   return hipGetLastError();
 }
 

@@ -208,22 +208,35 @@ inline Result<Array> dequantize(const Array &w, const Array &scales, const Array
 }
 
 // quantized_matmul(x, w, scales, biases, transpose, group_size, bits): x bf16 [M, K]; w u32
-// [N, K*bits/32] (transpose = false: [K, N*bits/32]); returns bf16 [M, N].  The reference's default is
-// transpose = false; the transposed layout (the one QuantizedLinear uses) is the tuned one and the
-// default here.
+// [N, K*bits/32] with transpose = true, [K, N*bits/32] without; scales and biases [N, K/group_size] /
+// [K, N/group_size]; returns bf16 [M, N].  transpose defaults to false as in the reference
+// (mlx-rs/src/ops/quantization.rs:101); QuantizedLinear passes true (nn/quantized.rs:363-386).
+// The operand shapes are checked against each other before anything is launched.
 inline Result<Array> quantized_matmul(const Array &x, const Array &w, const Array &scales,
                                       const Array *biases = nullptr, std::optional<bool> transpose = {},
                                       std::optional<int32_t> group_size = {},
                                       std::optional<int32_t> bits = {}, Stream s = {}) {
-  const bool tr = transpose.value_or(true);
+  const bool tr = transpose.value_or(false);
   const int32_t g = group_size.value_or(DEFAULT_GROUP_SIZE), b = bits.value_or(DEFAULT_BITS);
   if (auto e = detail::want(x, Dtype::Bfloat16, "quantized_matmul", "x")) return *e;
   if (auto e = detail::want(w, Dtype::Uint32, "quantized_matmul", "w")) return *e;
   if (auto e = detail::want(scales, Dtype::Bfloat16, "quantized_matmul", "scales")) return *e;
   if (!biases) return Exception("quantized_matmul: biases are required in affine mode");
   if (x.ndim() != 2 || w.ndim() != 2) return Exception("quantized_matmul: x must be [M, K] and w [N, K*bits/32]");
+  if (auto e = detail::want(*biases, Dtype::Bfloat16, "quantized_matmul", "biases")) return *e;
   const int64_t M = x.dim(0);
+  if (b != 2 && b != 4 && b != 8) return Exception("quantized_matmul: bits must be 2, 4 or 8");
+  if (g != 32 && g != 64 && g != 128) return Exception("quantized_matmul: group_size must be 32, 64 or 128");
   const int32_t K = (int32_t)x.dim(1), N = tr ? (int32_t)w.dim(0) : (int32_t)(w.dim(1) * 32 / b);
+  const int64_t w_k = tr ? w.dim(1) * 32 / b : w.dim(0);
+  if (w_k != K)
+    return Exception("quantized_matmul: x has K = " + std::to_string(K) + ", w has K = " + std::to_string(w_k) +
+                     (tr ? " (transpose = true)" : " (transpose = false)"));
+  const int64_t q_rows = tr ? N : K, q_axis = tr ? K : N;
+  if (q_axis % g == 0 && (scales.ndim() != 2 || biases->ndim() != 2 || scales.dim(0) != q_rows || scales.dim(1) != q_axis / g ||
+                          biases->dim(0) != q_rows || biases->dim(1) != q_axis / g))
+    return Exception("quantized_matmul: scales and biases must be [" + std::to_string(q_rows) + ", " +
+                     std::to_string(q_axis / g) + "]");
   size_t ws_bytes = 0;
   if (mi_moe_quantized_matmul_workspace_size(M, K, b, &ws_bytes)) return detail::last_error("quantized_matmul");
   auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);
@@ -333,6 +346,32 @@ inline Result<Array> gather_qmm(const Array &x, const Array &w, const Array &sca
   for (int64_t d : wb_shape) E *= d;
   const int32_t M = (int32_t)x.dim(-2), K = (int32_t)x.dim(-1);
   const int32_t N = tr ? (int32_t)w.dim(-2) : (int32_t)(w.dim(-1) * 32 / b);
+  // index arrays of one shape need no broadcast: they go to the library as they are, on the device
+  if (lhs_indices && rhs_indices && lhs_indices->shape() == rhs_indices->shape()) {
+    if (lhs_indices->dtype() != Dtype::Uint32 || rhs_indices->dtype() != Dtype::Uint32)
+      return Exception("gather_qmm: index arrays must be uint32");
+    const int64_t n_same = rhs_indices->size();
+    std::vector<int64_t> shape_same = rhs_indices->shape();
+    shape_same.push_back(M);
+    shape_same.push_back(N);
+    auto y = Array::empty(shape_same, x.dtype());
+    if (y.is_err() || n_same == 0) return y;
+    size_t wb = 0;
+    if (mi_moe_gather_qmm_workspace_size((int32_t)std::min<int64_t>(std::max<int64_t>(E, 1), 512), n_same, M, &wb))
+      return detail::last_error("gather_qmm");
+    auto ws = Array::empty({(int64_t)(wb + 256 + 3) / 4}, Dtype::Uint32);
+    if (ws.is_err()) return ws;
+    const int rc = mi_moe_gather_qmm_typed(x.data(), w.ptr<uint32_t>(), scales.data(), biases->data(),
+                                           lhs_indices->ptr<uint32_t>(), rhs_indices->ptr<uint32_t>(), n_same, xb, M, N, K,
+                                           (int32_t)E, tr ? 1 : 0, g, b, sorted ? 1 : 0, dt, y.value().data(),
+                                           ws.value().data(), ws.value().nbytes(), s.as_ptr());
+    // the workspace goes when this function returns: the work that uses it must have finished (also after a failure)
+    const hipError_t e = hipStreamSynchronize(s.handle);
+    if (rc) return detail::last_error("gather_qmm");
+    if (e != hipSuccess) return detail::hip_error("gather_qmm", e);
+    return y;
+  }
+  // otherwise the arrays pass through the host, where they are broadcast (this path synchronises the stream)
   auto lh = idx::host_indices(lhs_indices, xb_shape, s);
   if (lh.is_err()) return lh.error();
   auto rh = idx::host_indices(rhs_indices, wb_shape, s);
@@ -349,22 +388,26 @@ inline Result<Array> gather_qmm(const Array &x, const Array &w, const Array &sca
   if (y.is_err() || n_idx == 0) return y;
   auto ld = Array::from_host(lf.data(), {n_idx}, Dtype::Uint32, s);
   auto rd = Array::from_host(rf.data(), {n_idx}, Dtype::Uint32, s);
-  if (ld.is_err()) return ld;
-  if (rd.is_err()) return rd;
+  // from here on the uploads of the index copies may be in flight: every way out waits for the stream
+  // before the copies (and the workspace) are released
+  auto leave = [&](Result<Array> r) -> Result<Array> {
+    const hipError_t e = hipStreamSynchronize(s.handle);
+    if (r.is_err() || e == hipSuccess) return r;
+    return detail::hip_error("gather_qmm", e);
+  };
+  if (ld.is_err()) return leave(ld);
+  if (rd.is_err()) return leave(rd);
   size_t ws_bytes = 0;
   if (mi_moe_gather_qmm_workspace_size((int32_t)std::min<int64_t>(std::max<int64_t>(E, 1), 512), n_idx, M, &ws_bytes))
-    return detail::last_error("gather_qmm");
+    return leave(detail::last_error("gather_qmm"));
   auto ws = Array::empty({(int64_t)(ws_bytes + 256 + 3) / 4}, Dtype::Uint32);
-  if (ws.is_err()) return ws;
+  if (ws.is_err()) return leave(ws);
   if (mi_moe_gather_qmm_typed(x.data(), w.ptr<uint32_t>(), scales.data(), biases->data(), ld.value().ptr<uint32_t>(),
                               rd.value().ptr<uint32_t>(), n_idx, xb, M, N, K, (int32_t)E, tr ? 1 : 0, g, b,
                               sorted ? 1 : 0, dt, y.value().data(), ws.value().data(), ws.value().nbytes(),
                               s.as_ptr()))
-    return detail::last_error("gather_qmm");
-  // the workspace and the index copies may be released only after the work that uses them has finished
-  if (hipError_t e = hipStreamSynchronize(s.handle); e != hipSuccess)
-    return detail::hip_error("gather_qmm", e);
-  return y;
+    return leave(detail::last_error("gather_qmm"));
+  return leave(y);
 }
 
 }  // namespace ops

@@ -90,10 +90,22 @@ class SparseMoeBlock:
         the residual add behind it (mlx-lm/src/models/qwen3.rs:310-325) in one call."""
         return self.forward(x, debug=debug, out=out, _norm=(_need(norm_weight, torch.bfloat16, "norm_weight"), eps))
 
+    @staticmethod
+    def _check_out(out, x2, who):
+        """`out` is written through its raw pointer: it must be what the kernels assume."""
+        _need(out, torch.bfloat16, "out")
+        if out.device != x2.device:
+            raise capi.MoeError(f"{who}: out is on {out.device}, x on {x2.device}")
+        if out.numel() != x2.numel():
+            raise capi.MoeError(f"{who}: out must hold {x2.numel()} elements, got {out.numel()}")
+        return out
+
     def forward_static(self, x, out=None):
         """forward() on the library's built-in scratch instead of a workspace tensor
         (mi_moe_forward_static): nothing is allocated by the call when ``out`` is given.  Raises
-        when the batch needs more workspace than the scratch holds."""
+        when the batch needs more workspace than the scratch holds.  Every call on one GPU, through
+        whatever block, uses the same scratch array: calls that overlap on a GPU (two streams, two
+        threads) race, so keep them on one stream or order them with events."""
         _need(x, torch.bfloat16, "x")
         c = self.config
         if x.shape[-1] != c.hidden:
@@ -101,6 +113,8 @@ class SparseMoeBlock:
         x2 = x.reshape(-1, c.hidden)
         if out is None:
             out = torch.empty_like(x2)
+        else:
+            self._check_out(out, x2, "forward_static")
         check(self._lib.mi_moe_forward_static(self._handle, _ptr(x2), x2.shape[0], _ptr(out), None, _stream()))
         return out.reshape(x.shape)
 
@@ -115,6 +129,8 @@ class SparseMoeBlock:
         T = x2.shape[0]
         if out is None:
             out = torch.empty_like(x2)
+        else:
+            self._check_out(out, x2, "forward")
         ws = self.reserve(max(T, 1))
         dbg_struct, dbg = None, None
         if debug:
@@ -149,6 +165,8 @@ class SparseMoeBlock:
         T = x2.shape[0]
         if out is None:
             out = torch.empty_like(x2)
+        else:
+            self._check_out(out, x2, "forward_timed")
         ws = self.reserve(max(T, 1))
         ms = (C.c_float * capi.N_STAGES)()
         kms = (C.c_float * capi.N_KERNEL_TIMES)()

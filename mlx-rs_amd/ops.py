@@ -68,18 +68,29 @@ def quantize(w, group_size=64, bits=4, dtype=torch.bfloat16):
     return q, s, b
 
 
-def dequantize(w_q, scales, biases, group_size=64, bits=4):
-    """ops::dequantize (mlx-rs/src/ops/quantization.rs:124-158), fp32 result; scales and biases in
-    bfloat16, float16 or float32."""
+def dequantize(w_q, scales, biases, group_size=64, bits=4, dtype=None):
+    """ops::dequantize (mlx-rs/src/ops/quantization.rs:124-158); scales and biases in bfloat16,
+    float16 or float32.  The result has their element type, as the reference's has; ``dtype=torch.float32``
+    asks for the fp32 values before that last rounding."""
     lib = load_library()
     _need(w_q, torch.int32, "w_q")
     dt = _float_dtype(scales, "scales")
     _need(biases, scales.dtype, "biases")
+    if dtype is None:
+        dtype = scales.dtype
+    if dtype not in (scales.dtype, torch.float32):
+        raise capi.MoeError(f"dequantize: dtype must be that of the scales ({scales.dtype}) or float32, got {dtype}")
+    if w_q.dim() != 2:
+        raise capi.MoeError("dequantize: w_q must be a matrix")
     rows = w_q.shape[0]
     cols = w_q.shape[1] * 32 // bits
-    out = torch.empty((rows, cols), dtype=torch.float32, device=w_q.device)
-    check(lib.mi_moe_dequantize_typed(_ptr(w_q), _ptr(scales), _ptr(biases), rows, cols, group_size, bits, dt,
-                                      _ptr(out), _stream()))
+    if group_size > 0 and cols % group_size == 0 and tuple(scales.shape) != (rows, cols // group_size):
+        raise capi.MoeError(f"dequantize: scales must be [{rows}, {cols // group_size}], got {tuple(scales.shape)}")
+    if biases.shape != scales.shape:
+        raise capi.MoeError("dequantize: biases must have the shape of scales")
+    out = torch.empty((rows, cols), dtype=dtype, device=w_q.device)
+    fn = lib.mi_moe_dequantize_typed if dtype == torch.float32 else lib.mi_moe_dequantize_native
+    check(fn(_ptr(w_q), _ptr(scales), _ptr(biases), rows, cols, group_size, bits, dt, _ptr(out), _stream()))
     return out
 
 
@@ -114,6 +125,9 @@ def gather_qmm(x, w, scales, biases, lhs_indices=None, rhs_indices=None, transpo
     kw = w.shape[-1] * 32 // bits if transpose else w.shape[-2]
     if kw != K:
         raise capi.MoeError(f"gather_qmm: x has K = {K}, w has K = {kw}")
+    if scales.dim() != w.dim() or biases.dim() != w.dim():
+        raise capi.MoeError("gather_qmm: scales and biases must have as many axes as w")
+    _check_qmat("gather_qmm", w, scales, biases, K, transpose, group_size, bits)
     dev = x.device
 
     def counted(shape):
@@ -141,29 +155,71 @@ def gather_qmm(x, w, scales, biases, lhs_indices=None, rhs_indices=None, transpo
     return y.reshape(*out_batch, M, N)
 
 
-def quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4):
-    """ops::quantized_matmul (mlx-rs/src/ops/quantization.rs:91-122) the way QuantizedLinear calls
-    it (transpose = true, mlx-rs/src/nn/quantized.rs:363-386): x: [..., K] in bfloat16, float16 or
-    float32 (scales and biases in the same type); w: int32 [N, K*bits/32]; returns [..., N].
-    transpose = False (the op's own default): w int32 [K, N*bits/32], scales/biases [K, N/group_size]."""
+def _check_qmat(who, w, scales, biases, K, transpose, group_size, bits):
+    """Shapes of one quantized matrix against x's K: returns N.  w [N, K*bits/32] and scales / biases
+    [N, K/group_size] with transpose, w [K, N*bits/32] and scales / biases [K, N/group_size] without."""
+    if bits not in (2, 4, 8) or group_size not in (32, 64, 128):
+        return None  # the library words the refusal
+    per = 32 // bits
+    if transpose:
+        N, kw = w.shape[-2], w.shape[-1] * per
+    else:
+        N, kw = w.shape[-1] * per, w.shape[-2]
+    if kw != K:
+        raise capi.MoeError(f"{who}: x has K = {K}, w has K = {kw} (transpose = {bool(transpose)}, w {tuple(w.shape)})")
+    rows, q_axis = (N, K) if transpose else (K, N)
+    if q_axis % group_size == 0:
+        want = (rows, q_axis // group_size)
+        for t, name in ((scales, "scales"), (biases, "biases")):
+            if tuple(t.shape[-2:]) != want or tuple(t.shape[:-2]) != tuple(w.shape[:-2]):
+                raise capi.MoeError(f"{who}: {name} must be {tuple(w.shape[:-2]) + want}, got {tuple(t.shape)}")
+    return N
+
+
+def quantized_matmul(x, w, scales, biases, transpose=False, group_size=64, bits=4):
+    """ops::quantized_matmul (mlx-rs/src/ops/quantization.rs:91-122), same argument order and defaults
+    (``transpose`` defaults to False as there; QuantizedLinear passes True, mlx-rs/src/nn/quantized.rs:363-386).
+    x: [..., K] in bfloat16, float16 or float32 (scales and biases in the same type).
+    transpose = True: w int32 [N, K*bits/32], scales/biases [N, K/group_size];
+    transpose = False: w int32 [K, N*bits/32], scales/biases [K, N/group_size].  Returns [..., N]."""
+    return quantized_linear(x, w, scales, biases, None, transpose, group_size, bits, _who="quantized_matmul")
+
+
+def quantized_linear(x, w, scales, biases, linear_bias=None, transpose=True, group_size=64, bits=4,
+                     _who="quantized_linear"):
+    """QuantizedLinear::forward (mlx-rs/src/nn/quantized.rs:363-386): quantized_matmul with
+    transpose = True, then ``+ linear_bias`` ([N], x's type) when the layer has one; each of the two
+    ops rounds to x's type, as the reference's."""
     lib = load_library()
     dt = _float_dtype(x, "x")
     _need(w, torch.int32, "w")
     _need(scales, x.dtype, "scales")
     _need(biases, x.dtype, "biases")
-    if w.dim() != 2 or x.dim() < 1:
-        raise capi.MoeError("quantized_matmul: x must be [..., K] and w [N, K*bits/32]")
+    if w.dim() != 2 or x.dim() < 1 or scales.dim() != 2 or biases.dim() != 2:
+        raise capi.MoeError(f"{_who}: x must be [..., K], w, scales and biases matrices")
     K = x.shape[-1]
-    N = w.shape[0] if transpose else w.shape[1] * 32 // bits
+    N = _check_qmat(_who, w, scales, biases, K, transpose, group_size, bits)
+    if N is None:
+        N = w.shape[0] if transpose else w.shape[1] * 32 // max(bits, 1)
+    if linear_bias is not None:
+        if not transpose:
+            raise capi.MoeError(f"{_who}: a linear bias goes with transpose = True (the layout of QuantizedLinear)")
+        _need(linear_bias, x.dtype, "linear_bias")
+        if linear_bias.numel() != N:
+            raise capi.MoeError(f"{_who}: linear_bias must have {N} elements, got {linear_bias.numel()}")
     x2 = x.reshape(-1, K)
     M = x2.shape[0]
     y = torch.empty((M, N), dtype=x.dtype, device=x.device)
     need = C.c_size_t()
     check(lib.mi_moe_quantized_matmul_workspace_size(M, K, bits, C.byref(need)))
     ws = _workspace(need.value, x.device)
-    check(lib.mi_moe_quantized_matmul_typed(_ptr(x2), _ptr(w), _ptr(scales), _ptr(biases), M, N, K,
-                                            1 if transpose else 0, group_size, bits, dt, _ptr(y), _ptr(ws),
-                                            ws.numel(), _stream()))
+    if linear_bias is None:
+        check(lib.mi_moe_quantized_matmul_typed(_ptr(x2), _ptr(w), _ptr(scales), _ptr(biases), M, N, K,
+                                                1 if transpose else 0, group_size, bits, dt, _ptr(y), _ptr(ws),
+                                                ws.numel(), _stream()))
+    else:
+        check(lib.mi_moe_quantized_linear_typed(_ptr(x2), _ptr(w), _ptr(scales), _ptr(biases), _ptr(linear_bias), M, N, K,
+                                                group_size, bits, dt, _ptr(y), _ptr(ws), ws.numel(), _stream()))
     return y.reshape(*x.shape[:-1], N)
 
 

@@ -102,6 +102,16 @@ extern "C" {
     pub fn mi_moe_quantize_typed(w: *const f32, rows: i64, cols: i64, group_size: i32, bits: i32, dtype: i32, q: *mut u32, scales: *mut c_void, biases: *mut c_void, stream: *mut c_void) -> c_int;
     pub fn mi_moe_dequantize_typed(q: *const u32, scales: *const c_void, biases: *const c_void, rows: i64, cols: i64, group_size: i32, bits: i32, dtype: i32, w_hat: *mut f32, stream: *mut c_void) -> c_int;
 
+    pub fn mi_moe_quantized_linear_typed(x: *const c_void, w: *const u32, scales: *const c_void, biases: *const c_void, linear_bias: *const c_void, M: i64, N: i32, K: i32, group_size: i32, bits: i32, dtype: i32, y: *mut c_void, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
+    pub fn mi_moe_dequantize_native(q: *const u32, scales: *const c_void, biases: *const c_void, rows: i64, cols: i64, group_size: i32, bits: i32, dtype: i32, w_hat: *mut c_void, stream: *mut c_void) -> c_int;
+
+    pub fn mi_moe_debug_kernel_count() -> i32;
+    pub fn mi_moe_debug_kernel_name(index: i32) -> *const c_char;
+    pub fn mi_moe_debug_kernel_launches(index: i32) -> i64;
+    pub fn mi_moe_debug_plan_forward(cfg: *const mi_moe_config, T: i64, out: *mut c_char, cap: usize) -> c_int;
+    pub fn mi_moe_debug_plan_grouped(N: i32, K: i32, bits: i32, glu: i32, total_rows: i64, max_active: i32, max_rows_per_expert: i64, max_streamed_rows: i64, tile_lists: i32, paired_out: i32, out: *mut c_char, cap: usize) -> c_int;
+    pub fn mi_moe_debug_side_streams_created() -> i32;
+
     pub fn mi_moe_stream_probe(buf: *const c_void, bytes: usize, sink: *mut u32, stream: *mut c_void) -> c_int;
 
     pub fn mi_moe_version() -> *const c_char;

@@ -98,6 +98,122 @@ pub mod ops {
         Ok((q, s, b))
     }
 
+    /// The quantisation mode of the reference's ops (`DEFAULT_MODE`, what `mlx-rs/src/ops/quantization.rs:213-227`
+    /// hands to `mlx_gather_qmm` / `mlx_quantized_matmul` / `mlx_quantize`).  This library implements this mode only.
+    pub const DEFAULT_MODE: &str = "affine";
+
+    /// Refuses every mode but `"affine"`, in the shape of an MLX error.  The `*_with_mode` functions below
+    /// stand where a caller of the `-sys` level passes a mode string.
+    pub fn check_mode(mode: impl Into<Option<&'static str>>, op: &str) -> Result<(), Exception> {
+        match mode.into().unwrap_or(DEFAULT_MODE) {
+            "affine" => Ok(()),
+            other => Err(Exception::custom(format!(
+                "[{op}] Invalid quantization mode '{other}': mi_moe implements the 'affine' mode only (one scale and one bias per group)"
+            ))),
+        }
+    }
+
+    /// `gather_qmm` with the `mode` argument of `mlx_gather_qmm`; anything but `"affine"` is an error.
+    #[allow(clippy::too_many_arguments)]
+    pub fn gather_qmm_with_mode<'l, 'r, D: DeviceAccess>(
+        x: &Array,
+        w: &Array,
+        scales: &Array,
+        biases: &Array,
+        lhs_indices: impl Into<Option<&'l Array>>,
+        rhs_indices: impl Into<Option<&'r Array>>,
+        transpose: impl Into<Option<bool>>,
+        group_size: impl Into<Option<i32>>,
+        bits: impl Into<Option<i32>>,
+        mode: impl Into<Option<&'static str>>,
+        sorted_indices: impl Into<Option<bool>>,
+        stream: &Stream,
+    ) -> Result<Array, Exception> {
+        check_mode(mode, "gather_qmm")?;
+        gather_qmm::<D>(x, w, scales, biases, lhs_indices, rhs_indices, transpose, group_size, bits, sorted_indices, stream)
+    }
+
+    /// `quantized_matmul` with the `mode` argument of `mlx_quantized_matmul`; anything but `"affine"` is an error.
+    #[allow(clippy::too_many_arguments)]
+    pub fn quantized_matmul_with_mode<D: DeviceAccess>(
+        x: &Array,
+        w: &Array,
+        scales: &Array,
+        biases: &Array,
+        transpose: impl Into<Option<bool>>,
+        group_size: impl Into<Option<i32>>,
+        bits: impl Into<Option<i32>>,
+        mode: impl Into<Option<&'static str>>,
+        stream: &Stream,
+    ) -> Result<Array, Exception> {
+        check_mode(mode, "quantized_matmul")?;
+        quantized_matmul::<D>(x, w, scales, biases, transpose, group_size, bits, stream)
+    }
+
+    /// `QuantizedLinear::forward` (`mlx-rs/src/nn/quantized.rs:363-386`): `quantized_matmul(x, w, scales, biases,
+    /// true, ..)`, then `+ bias` when the layer has one (`mi_moe_quantized_linear_typed`).
+    #[allow(clippy::too_many_arguments)]
+    pub fn quantized_linear<'b, D: DeviceAccess>(
+        x: &Array,
+        w: &Array,
+        scales: &Array,
+        biases: &Array,
+        linear_bias: impl Into<Option<&'b Array>>,
+        group_size: impl Into<Option<i32>>,
+        bits: impl Into<Option<i32>>,
+        stream: &Stream,
+    ) -> Result<Array, Exception> {
+        let group_size = group_size.into().unwrap_or(DEFAULT_GROUP_SIZE);
+        let bits = bits.into().unwrap_or(DEFAULT_BITS);
+        let dt = float_code(x, "x")?;
+        expect_dtype(w, Dtype::Uint32, "w")?;
+        expect_dtype(scales, x.dtype(), "scales")?;
+        expect_dtype(biases, x.dtype(), "biases")?;
+        let linear_bias = linear_bias.into();
+        let (k, n) = (x.dim(-1), w.dim(-2));
+        if let Some(b) = linear_bias {
+            expect_dtype(b, x.dtype(), "bias")?;
+            if b.size() as i32 != n {
+                return Err(Exception::custom("[mi_moe] quantized_linear: the bias must have one element per output column"));
+            }
+        }
+        let m: i64 = x.shape()[..x.ndim() - 1].iter().map(|&d| d as i64).product();
+        let mut ws_bytes = 0usize;
+        check(unsafe { sys::mi_moe_quantized_matmul_workspace_size(m, k, bits, &mut ws_bytes) })?;
+        let mut ws = D::device_buffer(ws_bytes.max(256))?;
+        let mut shape = x.shape().to_vec();
+        *shape.last_mut().unwrap() = n;
+        let mut y = empty_like_dtype(x, &shape)?;
+        check(unsafe {
+            sys::mi_moe_quantized_linear_typed(D::device_ptr(x), D::device_ptr(w) as *const u32, D::device_ptr(scales), D::device_ptr(biases), linear_bias.map_or(std::ptr::null(), |b| D::device_ptr(b)), m, n, k, group_size, bits, dt, D::device_ptr_mut(&mut y), D::device_ptr_mut(&mut ws), ws_bytes, D::hip_stream(stream))
+        })?;
+        Ok(y)
+    }
+
+    /// `ops::dequantize` as the reference returns it (`mlx-rs/src/ops/quantization.rs:124-158`): the result has
+    /// the element type of `scales` (`mi_moe_dequantize_native`).
+    pub fn dequantize_native<D: DeviceAccess>(
+        w: &Array,
+        scales: &Array,
+        biases: &Array,
+        group_size: impl Into<Option<i32>>,
+        bits: impl Into<Option<i32>>,
+        stream: &Stream,
+    ) -> Result<Array, Exception> {
+        let group_size = group_size.into().unwrap_or(DEFAULT_GROUP_SIZE);
+        let bits = bits.into().unwrap_or(DEFAULT_BITS);
+        expect_dtype(w, Dtype::Uint32, "w")?;
+        let dt = float_code(scales, "scales")?;
+        expect_dtype(biases, scales.dtype(), "biases")?;
+        let rows = w.dim(-2) as i64;
+        let cols = w.dim(-1) as i64 * 32 / bits as i64;
+        let mut out = empty_like_dtype(scales, &[rows as i32, cols as i32])?;
+        check(unsafe {
+            sys::mi_moe_dequantize_native(D::device_ptr(w) as *const u32, D::device_ptr(scales), D::device_ptr(biases), rows, cols, group_size, bits, dt, D::device_ptr_mut(&mut out), D::hip_stream(stream))
+        })?;
+        Ok(out)
+    }
+
     /// `mi_moe_dequantize_typed`: float32 `[rows, cols]`; scales and biases in any floating type.
     pub fn dequantize<D: DeviceAccess>(
         w: &Array,

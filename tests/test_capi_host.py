@@ -139,3 +139,29 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(m.capi, "_SO", "/nonexistent/libmi_moe.so")
     with pytest.raises(m.MoeError):
         m.capi.load_library()
+
+
+def test_operand_shapes_of_a_quantized_product_are_checked_on_the_host():
+    """The shape check of ops.quantized_matmul / gather_qmm (no GPU needed: shapes only).  The reference's
+    default is transpose = false (mlx-rs/src/ops/quantization.rs:101): a [N, K*bits/32] matrix handed over
+    without transpose = true is refused, not read as [K, N'*bits/32]."""
+    import inspect
+
+    import torch
+
+    from mlx_rs_amd import capi, ops
+    assert inspect.signature(ops.quantized_matmul).parameters["transpose"].default is False
+    assert inspect.signature(ops.gather_qmm).parameters["transpose"].default is True   # ops/quantization.rs:193
+    N, K = 64, 256
+    w = torch.empty((N, K // 8), dtype=torch.int32, device="meta")
+    s = torch.empty((N, K // 64), dtype=torch.bfloat16, device="meta")
+    assert ops._check_qmat("quantized_matmul", w, s, s, K, True, 64, 4) == N
+    with pytest.raises(capi.MoeError, match="K = 256, w has K = 64"):
+        ops._check_qmat("quantized_matmul", w, s, s, K, False, 64, 4)
+    with pytest.raises(capi.MoeError, match="scales must be"):
+        ops._check_qmat("quantized_matmul", w, s[:, :-1], s, K, True, 64, 4)
+    wn = torch.empty((K, N // 8), dtype=torch.int32, device="meta")
+    sn = torch.empty((K, N // 64), dtype=torch.bfloat16, device="meta")
+    assert ops._check_qmat("quantized_matmul", wn, sn, sn, K, False, 64, 4) == N
+    with pytest.raises(capi.MoeError, match="biases must be"):
+        ops._check_qmat("quantized_matmul", wn, sn, s, K, False, 64, 4)

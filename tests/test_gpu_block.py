@@ -288,3 +288,22 @@ def test_one_expert_is_the_dense_quantized_mlp(orc, bits, T):
     h = m.ops.swiglu(g, u)
     y = m.ops.quantized_matmul(h, *mats["down"], True, 64, bits)
     assert_close_bf16(got, bits_u16(y), what="block vs the chain of quantized_matmul and swiglu")
+
+
+def test_side_streams_belong_to_the_gpu_not_to_a_handle():
+    """A hundred handles on one GPU: no stream is created after the first handle's three, and a
+    prefill-sized forward through the last handle gives the first one's result."""
+    import mlx_rs_amd as m
+    from mlx_rs_amd import synth
+    lib = m.load_library()
+    cfg = m.MoeConfig(256, 8, 2, 512)
+    first = synth.make_block(cfg, seed=2, device="cuda", gen_device="cuda")
+    created = lib.mi_moe_debug_side_streams_created()
+    assert created >= 3 and created % 3 == 0
+    blocks = [m.SparseMoeBlock(cfg, first.gate_weight, first.gate_proj, first.up_proj, first.down_proj) for _ in range(100)]
+    assert lib.mi_moe_debug_side_streams_created() == created
+    x = synth.make_tokens(cfg, 512, seed=2, device="cuda")   # 128 rows per expert: tile classes on the side streams
+    a, b = first.forward(x), blocks[-1].forward(x)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert lib.mi_moe_debug_side_streams_created() == created

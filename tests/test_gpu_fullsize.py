@@ -44,6 +44,65 @@ CASES = [
 
 MIN_ORACLE_TOKENS = 512
 
+# Share of the compared elements that may lie beyond the flat 2e-2 (they are then held by the row-scaled
+# rule of helpers.py).  Zero for the shapes whose outputs stay within [-1, 1]; the Mixtral-shaped layer's
+# outputs reach |11| (one bf16 ulp of a value in [8, 16) is 6.25e-2), measured share 6.4 %.
+OVER_FLAT_CEILING = {"mixtral_8x7b": 0.10}
+
+# Shapes whose outputs exceed a flat 2e-2 against the op-by-op oracle are also compared with the
+# mathematics itself: the block recomputed in float64 from the definitions (no intermediate rounding),
+# with the routing and the bf16 scores taken as given.  The HIP result must be as close to that truth as
+# the oracle's op-by-op result is (which rounds after every MLX op), in max-abs and in relative
+# Frobenius error, and every element must lie within a few bf16 ulps of its row's scale of the truth.
+FP64_CHECKED = {"mixtral_8x7b"}
+FP64_ERR_VS_ORACLE = 1.25   # err(HIP, fp64) <= this * err(op-by-op oracle, fp64)
+FP64_ULPS_OF_ROW = 1.5      # |HIP - fp64| <= this many bf16 ulps of the row's largest |fp64| value
+
+
+def _dequant_fp64(bank, e, bits):
+    """float64 [N, K] of expert e, from the format's definition (codes low bits first, one scale and
+    bias per 64 codes), on the device."""
+    w = bank.weight[e].to(torch.int64) & 0xFFFFFFFF
+    per = 32 // bits
+    sh = torch.arange(per, device=w.device, dtype=torch.int64) * bits
+    q = ((w.unsqueeze(-1) >> sh) & ((1 << bits) - 1)).reshape(w.shape[0], -1).to(torch.float64)
+    sc = bank.scales[e].to(torch.float64).repeat_interleave(64, dim=1)
+    bi = bank.biases[e].to(torch.float64).repeat_interleave(64, dim=1)
+    return sc * q + bi
+
+
+def _check_against_fp64(blk, cfg, x, dbg, pick, got_bits, oracle_bits, what):
+    T, k = dbg["topk_idx"].shape
+    pick_t = torch.from_numpy(pick).cuda()
+    xs = x[pick_t].to(torch.float64)
+    idx = dbg["topk_idx"][pick_t].to(torch.int64)
+    sc = dbg["topk_w"][pick_t].to(torch.float64)
+    truth = torch.zeros((len(pick), cfg.hidden), dtype=torch.float64, device="cuda")
+    for e in range(cfg.n_experts):
+        rows, slots = torch.nonzero(idx == e, as_tuple=True)
+        if rows.numel() == 0:
+            continue
+        g = xs[rows] @ _dequant_fp64(blk.gate_proj, e, cfg.bits).T
+        u = xs[rows] @ _dequant_fp64(blk.up_proj, e, cfg.bits).T
+        h = g / (1.0 + torch.exp(-g)) * u
+        y = h @ _dequant_fp64(blk.down_proj, e, cfg.bits).T
+        truth.index_add_(0, rows, y * sc[rows, slots].unsqueeze(1))
+    truth = truth.cpu().numpy()
+    from helpers import f32_of_bits
+    got = f32_of_bits(got_bits).astype(np.float64)
+    orc_out = f32_of_bits(oracle_bits).astype(np.float64)
+    err_got, err_orc = np.abs(got - truth), np.abs(orc_out - truth)
+    fro = lambda d: float(np.linalg.norm(d) / np.linalg.norm(truth))
+    row_max = np.abs(truth).max(axis=1, keepdims=True)
+    ulp_row = 2.0 ** (np.floor(np.log2(np.maximum(row_max, 2.0 ** -126))) - 7)
+    ulps = err_got / ulp_row
+    print(f"  {what} vs float64: HIP max-abs {err_got.max():.3e} rel-Frobenius {fro(got - truth):.3e}; op-by-op oracle "
+          f"max-abs {err_orc.max():.3e} rel-Frobenius {fro(orc_out - truth):.3e}; HIP worst element {ulps.max():.2f} bf16 ulps "
+          f"of its row's scale (oracle {(err_orc / ulp_row).max():.2f}); max |truth| {np.abs(truth).max():.2f}", flush=True)
+    assert err_got.max() <= FP64_ERR_VS_ORACLE * err_orc.max()
+    assert fro(got - truth) <= FP64_ERR_VS_ORACLE * fro(orc_out - truth)
+    assert ulps.max() <= FP64_ULPS_OF_ROW
+
 
 def _plan(cfg, T):
     """Which segments the block tiles at this batch size: (tile lists built, rows from which a segment
@@ -164,4 +223,7 @@ def test_full_size_properties(orc, name, T, zipf):
     ref, d = orc.moe_forward(ocfg, W, xs, strict=True, n_threads=16)
     assert np.array_equal(d["topk_idx"].astype(np.int64), idx[pick]), "selection differs from the oracle"
     assert np.array_equal(d["topk_w"], bits_u16(dbg["topk_w"]).reshape(T, k)[pick]), "scores differ from the oracle"
-    assert_close_bf16(bits_u16(out)[pick], ref, what=f"{name} T={T}, {S} tokens vs oracle")
+    assert_close_bf16(bits_u16(out)[pick], ref, what=f"{name} T={T}, {S} tokens vs oracle",
+                      max_over_flat=OVER_FLAT_CEILING.get(name, 0.0))
+    if name in FP64_CHECKED:
+        _check_against_fp64(blk, cfg, x, dbg, pick, bits_u16(out)[pick], ref, f"{name} T={T}")

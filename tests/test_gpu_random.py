@@ -50,7 +50,7 @@ def test_random_gather_qmm_and_quantized_matmul_against_float64(m, seed):
         tag = f"draw {case}: bits={bits} M={M} N={N} K={K} E={E} n_idx={n_idx} x batch={xb} skewed={skew}"
         w = torch.randn(E * N, K, device="cuda") * 0.05
         q, s, b = m.ops.quantize(w, 64, bits)
-        w_hat = m.ops.dequantize(q, s, b, 64, bits).reshape(E, N, K)
+        w_hat = m.ops.dequantize(q, s, b, 64, bits, dtype=torch.float32).reshape(E, N, K)
         q, s, b = q.reshape(E, N, -1), s.reshape(E, N, -1), b.reshape(E, N, -1)
         x = torch.randn(xb, M, K, device="cuda").to(torch.bfloat16)
         if skew:

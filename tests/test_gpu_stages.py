@@ -145,13 +145,17 @@ def test_quantize_dequantize_bit_exact(orc, m, bits, group):
     q, s, b = orc.quantize(w, bits, group)
     gq, gs, gb = m.ops.quantize(torch.from_numpy(w).cuda(), group, bits)
     assert np.array_equal(bits_u32(gq), q) and np.array_equal(bits_u16(gs), s) and np.array_equal(bits_u16(gb), b)
-    wh = m.ops.dequantize(gq, gs, gb, group, bits).cpu().numpy()
+    wh = m.ops.dequantize(gq, gs, gb, group, bits, dtype=torch.float32).cpu().numpy()
     assert np.array_equal(wh, orc.dequantize(q, s, b, bits, group))
+    # as the reference returns it (ops/quantization.rs:124-158): in the type of the scales, one more rounding
+    wn = m.ops.dequantize(gq, gs, gb, group, bits)
+    assert wn.dtype == torch.bfloat16
+    assert np.array_equal(bits_u16(wn), orc.f32_to_bf16(orc.dequantize(q, s, b, bits, group)))
     # the reference's known-answer case (ops/quantization.rs:298-315) on the device
     x = np.tile(np.arange(512, dtype=np.float32), (128, 1))
     gq, gs, gb = m.ops.quantize(torch.from_numpy(x).cuda(), 128, bits)
     assert tuple(gq.shape) == (128, 512 * bits // 32) and tuple(gs.shape) == (128, 4)
-    xh = m.ops.dequantize(gq, gs, gb, 128, bits).cpu().numpy()
+    xh = m.ops.dequantize(gq, gs, gb, 128, bits, dtype=torch.float32).cpu().numpy()
     assert np.abs(x - xh).max() <= 127.0 / (1 << bits) + 2.0   # + bf16 rounding of a bias near 511
 
 

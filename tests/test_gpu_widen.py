@@ -208,3 +208,47 @@ def test_indices_out_of_range_are_clamped_not_followed(m, dtype):
     rc = lib.mi_moe_gather_qmm(x.data_ptr(), qw.data_ptr(), sw.data_ptr(), bw.data_ptr(), None, rhs.data_ptr(), 3, 2, M, N, K,
                                4, 1, group_size, bits, 0, y.data_ptr(), None, 0, None)
     assert rc != 0 and b"need as many matrices in x" in lib.mi_moe_last_error()
+
+
+@pytest.mark.parametrize("dtype,bits,group,M", [(torch.bfloat16, 4, 64, 3), (torch.bfloat16, 8, 64, 300),
+                                                (torch.float32, 4, 128, 5), (torch.float16, 2, 32, 2)])
+def test_quantized_linear_adds_its_bias(m, dtype, bits, group, M):
+    """QuantizedLinear::forward (mlx-rs/src/nn/quantized.rs:363-386): quantized_matmul(transpose = true), then
+    `+ bias`.  Against the two ops done separately (bit for bit: the entry point rounds where they round) and
+    against float64."""
+    g = torch.Generator().manual_seed(bits * 10 + M)
+    N, K = 192, 256
+    w = (torch.randn((N, K), generator=g) * 0.05).cuda()
+    w_q, s, b = m.ops.quantize(w, group, bits, dtype=dtype)
+    x = torch.randn((M, K), generator=g).to(dtype).cuda()
+    lb = torch.randn((N,), generator=g).to(dtype).cuda()
+    y = m.ops.quantized_linear(x, w_q, s, b, lb, True, group, bits)
+    y0 = m.ops.quantized_matmul(x, w_q, s, b, True, group, bits)
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and tuple(y.shape) == (M, N)
+    assert torch.equal(y, (y0.float() + lb.float()).to(dtype)), "not the reference's two ops"
+    assert torch.equal(m.ops.quantized_linear(x, w_q, s, b, None, True, group, bits), y0)
+    w_hat = m.ops.dequantize(w_q, s, b, group, bits, dtype=torch.float32).double()
+    ref = x.double() @ w_hat.T + lb.double()
+    tol = 2e-2 if dtype == torch.bfloat16 else (4e-3 if dtype == torch.float16 else 1e-4)
+    assert (y.double() - ref).abs().max().item() <= tol * max(1.0, ref.abs().max().item())
+    with pytest.raises(m.capi.MoeError):
+        m.ops.quantized_linear(x, w_q, s, b, lb[:-1].contiguous(), True, group, bits)
+
+
+def test_operand_shapes_are_checked_against_each_other(m):
+    """A call in the reference's default layout (transpose = false, w [K, N*bits/32]) whose operands belong to
+    the other layout is refused by the host layer instead of being read past its ends."""
+    g = torch.Generator().manual_seed(1)
+    N, K = 64, 256
+    w_q, s, b = m.ops.quantize((torch.randn((N, K), generator=g) * 0.05).cuda(), 64, 4)  # [N, K/8]: the transposed layout
+    x = torch.randn((2, K), generator=g).to(torch.bfloat16).cuda()
+    with pytest.raises(m.capi.MoeError, match="K ="):
+        m.ops.quantized_matmul(x, w_q, s, b)               # default transpose = False, as the reference's
+    y = m.ops.quantized_matmul(x, w_q, s, b, True)
+    assert tuple(y.shape) == (2, N)
+    with pytest.raises(m.capi.MoeError, match="scales"):
+        m.ops.quantized_matmul(x, w_q, s[:, :-1].contiguous(), b[:, :-1].contiguous(), True)
+    with pytest.raises(m.capi.MoeError, match="scales"):
+        m.ops.gather_qmm(x.reshape(2, 1, K), w_q.reshape(1, N, -1), s.reshape(1, N, -1)[:, :-1].contiguous(),
+                         b.reshape(1, N, -1)[:, :-1].contiguous(), rhs_indices=torch.zeros(2, dtype=torch.int32, device="cuda"))

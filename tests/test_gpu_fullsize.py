@@ -46,17 +46,22 @@ MIN_ORACLE_TOKENS = 512
 
 # Share of the compared elements that may lie beyond the flat 2e-2 (they are then held by the row-scaled
 # rule of helpers.py).  Zero for the shapes whose outputs stay within [-1, 1]; the Mixtral-shaped layer's
-# outputs reach |11| (one bf16 ulp of a value in [8, 16) is 6.25e-2), measured share 6.4 %.
-OVER_FLAT_CEILING = {"mixtral_8x7b": 0.10}
+# outputs reach |11| (one bf16 ulp of a value in [8, 16) is 6.25e-2), measured share 6.4 %; the
+# Qwen3-235B-shaped layer's reach |3.3| with Zipf routing at a few hundred tokens (21 of 1.57 M elements).
+OVER_FLAT_CEILING = {"mixtral_8x7b": 0.10, "qwen3_235b_a22b": 1e-4}
 
 # Shapes whose outputs exceed a flat 2e-2 against the op-by-op oracle are also compared with the
 # mathematics itself: the block recomputed in float64 from the definitions (no intermediate rounding),
 # with the routing and the bf16 scores taken as given.  The HIP result must be as close to that truth as
 # the oracle's op-by-op result is (which rounds after every MLX op), in max-abs and in relative
-# Frobenius error, and every element must lie within a few bf16 ulps of its row's scale of the truth.
-FP64_CHECKED = {"mixtral_8x7b"}
-FP64_ERR_VS_ORACLE = 1.25   # err(HIP, fp64) <= this * err(op-by-op oracle, fp64)
-FP64_ULPS_OF_ROW = 1.5      # |HIP - fp64| <= this many bf16 ulps of the row's largest |fp64| value
+# Frobenius error and in its worst element, and every element must lie within a few bf16 ulps of its row's
+# scale of the truth.  Measured at 320 tokens (1.3 M elements, |truth| up to 11.3): HIP max-abs 5.6e-2,
+# rel-Frobenius 4.0e-3, worst element 1.73 ulps of its row's scale; op-by-op oracle 6.9e-2, 4.8e-3, 2.19 ulps:
+# the excess over a flat 2e-2 is bf16 rounding at this output scale, and the fused kernels carry less of it
+# than the op-by-op sequence.
+FP64_CHECKED = {"mixtral_8x7b", "qwen3_235b_a22b"}
+FP64_ERR_VS_ORACLE = 1.25   # err(HIP, fp64) <= this * err(op-by-op oracle, fp64): max-abs, rel-Frobenius, worst ulps
+FP64_ULPS_OF_ROW = 2.5      # |HIP - fp64| <= this many bf16 ulps of the row's largest |fp64| value
 
 
 def _dequant_fp64(bank, e, bits):
@@ -102,6 +107,7 @@ def _check_against_fp64(blk, cfg, x, dbg, pick, got_bits, oracle_bits, what):
     assert err_got.max() <= FP64_ERR_VS_ORACLE * err_orc.max()
     assert fro(got - truth) <= FP64_ERR_VS_ORACLE * fro(orc_out - truth)
     assert ulps.max() <= FP64_ULPS_OF_ROW
+    assert ulps.max() <= FP64_ERR_VS_ORACLE * (err_orc / ulp_row).max()
 
 
 def _plan(cfg, T):

@@ -83,30 +83,13 @@ def time_steps(fn, steps, warmup, torch):
     return (time.perf_counter() - t0) / steps * 1e3
 
 
-def tile_class_rows(counts, cfg, T):
+def tile_class_rows(counts, cfg, T, capi):
     """Rows of the batch that each grouped-product kernel processes: [256-row tiles, 128-row tiles,
-    64-row tiles, streamed], by the library's rule (segments of tmr rows and more are cut into 256-row
-    tiles, the remainder goes to the smallest class that holds it; shorter segments stream)."""
-    P, E = T * cfg.top_k, cfg.n_experts
-    light, heavy_avg = (6, 20) if cfg.bits == 4 else (17, 17)
-    even_groups = (cfg.hidden // 64) % 2 == 0 and (cfg.intermediate // 64) % 2 == 0
-    heavy = P >= heavy_avg * E
-    tiled = even_groups and (P >= light * E or heavy)
-    tmr = (9 if heavy else 17) if cfg.bits == 4 else 17
+    64-row tiles, streamed], by the library's own rule (capi.tile_rule, capi.segment_rows_by_kernel)."""
+    tiled, tmr = capi.tile_rule(cfg.c_struct(), T)
     rows = [0, 0, 0, 0]
     for c in counts:
-        c = int(c)
-        if not tiled or c < tmr:
-            rows[3] += c
-            continue
-        full, r = divmod(c, 256)
-        rows[0] += full * 256
-        if r > 128:
-            rows[0] += r
-        elif r > 64:
-            rows[1] += r
-        else:
-            rows[2] += r
+        rows = [a + b for a, b in zip(rows, capi.segment_rows_by_kernel(c, tiled, tmr))]
     return rows
 
 
@@ -144,7 +127,7 @@ def run_workload(name, args, torch, m, synth, dev):
             c = dbg["counts"].cpu().numpy()
             actives.append(int((c > 0).sum()))
             counts_stats.append((int(c.max()), float(c.mean()), int(c.min())))
-            class_rows.append(tile_class_rows(c, cfg, T))
+            class_rows.append(tile_class_rows(c, cfg, T, m.capi))
         n_active = sum(actives) / len(actives)
         class_rows = [sum(r[i] for r in class_rows) / len(class_rows) for i in range(4)]
 

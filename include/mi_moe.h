@@ -313,6 +313,10 @@ int mi_moe_debug_plan_grouped(int32_t N, int32_t K, int32_t bits, int32_t glu, i
                               int32_t max_active, int64_t max_rows_per_expert,
                               int64_t max_streamed_rows, int32_t tile_lists, int32_t paired_out,
                               char *out, size_t cap);
+/* which rows of a forward of T tokens go where: *tiled = M-tile lists are built; *tile_min_rows = a segment of
+ * at least that many rows is cut into 256-row tiles, with its remainder in the 256-, 128- or 64-row list that
+ * holds it; shorter segments stream */
+int mi_moe_debug_tile_rule(const mi_moe_config *cfg, int64_t T, int32_t *tiled, int32_t *tile_min_rows);
 int32_t mi_moe_debug_side_streams_created(void);
 
 /* ---- measurement aid; no counterpart in the reference.  A bare streaming kernel with the decode

@@ -29,7 +29,7 @@ EXPORTS = (
     "mi_moe_gather_qmm_typed", "mi_moe_quantized_matmul_typed", "mi_moe_quantize_typed", "mi_moe_dequantize_typed",
     "mi_moe_quantized_linear_typed", "mi_moe_dequantize_native",
     "mi_moe_debug_kernel_count", "mi_moe_debug_kernel_name", "mi_moe_debug_kernel_launches", "mi_moe_debug_plan_forward", "mi_moe_debug_plan_grouped",
-    "mi_moe_debug_side_streams_created",
+    "mi_moe_debug_side_streams_created", "mi_moe_debug_tile_rule",
 )
 
 
@@ -119,6 +119,7 @@ def load_library():
         "mi_moe_dequantize_native": [vp, vp, vp, i64, i64, i32, i32, i32, vp, vp],
         "mi_moe_quantized_linear_typed": [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, vp, sz, vp],
         "mi_moe_debug_plan_forward": [C.POINTER(Config), i64, C.c_char_p, sz],
+        "mi_moe_debug_tile_rule": [C.POINTER(Config), i64, C.POINTER(i32), C.POINTER(i32)],
         "mi_moe_debug_plan_grouped": [i32, i32, i32, i32, i64, i32, i64, i64, i32, i32, C.c_char_p, sz],
     }
     for name, args in sigs.items():
@@ -152,6 +153,31 @@ def _plan_entries(buf):
             name, *rest = item.split(" ")
             out.append((name, {k: v for k, v in (r.split("=") for r in rest)}))
     return out
+
+
+def tile_rule(cfg, tokens):
+    """(tile lists are built, rows from which a segment is tiled) for a forward of `tokens` tokens: the
+    library's own rule (needs no GPU)."""
+    tiled, tmr = C.c_int32(), C.c_int32()
+    check(load_library().mi_moe_debug_tile_rule(C.byref(cfg), tokens, C.byref(tiled), C.byref(tmr)))
+    return bool(tiled.value), tmr.value
+
+
+def segment_rows_by_kernel(count, tiled, tmr):
+    """Rows of a segment of `count` rows that each grouped-product kernel takes:
+    [256-row tiles, 128-row tiles, 64-row tiles, streamed] (see tile_rule)."""
+    count = int(count)
+    if not tiled or count < tmr:
+        return [0, 0, 0, count]
+    full, r = divmod(count, 256)
+    rows = [full * 256, 0, 0, 0]
+    if r > 128:
+        rows[0] += r
+    elif r > 64:
+        rows[1] = r
+    else:
+        rows[2] = r
+    return rows
 
 
 def plan_forward(cfg, tokens):

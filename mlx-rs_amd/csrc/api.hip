@@ -1049,6 +1049,15 @@ int mi_moe_debug_plan_forward(const mi_moe_config *cfg, int64_t T, char *out, si
   return 0;
 } MI_CATCH("debug_plan_forward")
 
+int mi_moe_debug_tile_rule(const mi_moe_config *cfg, int64_t T, int32_t *tiled, int32_t *tile_min_rows) try {
+  if (check_config(cfg)) return 1;
+  if (T < 0 || T * cfg->top_k > (int64_t)1 << 30) return fail("debug_tile_rule: token count out of range");
+  const ForwardWs f = carve_forward(*cfg, T, nullptr);
+  if (tiled) *tiled = f.tiled ? 1 : 0;
+  if (tile_min_rows) *tile_min_rows = f.tmr;
+  return 0;
+} MI_CATCH("debug_tile_rule")
+
 int32_t mi_moe_debug_side_streams_created(void) { return g_side_streams_created.load(); }
 
 }  // extern "C"

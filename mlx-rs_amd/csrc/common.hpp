@@ -18,14 +18,26 @@ constexpr int kWave = 64;
 // lists are not built.  Measured crossovers: see the design notes.
 #ifndef MI_TMR4
 #define MI_TMR4 9
+#endif
+#ifndef MI_TMR8
 #define MI_TMR8 17
+#endif
+#ifndef MI_TAVG4
 #define MI_TAVG4 20
+#endif
+#ifndef MI_TAVG8
 #define MI_TAVG8 17
 #endif
 #ifndef MI_TLIGHT4
 #define MI_TLIGHT4 6
+#endif
+#ifndef MI_TLIGHT8
 #define MI_TLIGHT8 17
+#endif
+#ifndef MI_TMRL4
 #define MI_TMRL4 17
+#endif
+#ifndef MI_TMRL8
 #define MI_TMRL8 17
 #endif
 __host__ __device__ constexpr int tile_min_rows(int bits, bool heavy) {

@@ -110,6 +110,7 @@ extern "C" {
     pub fn mi_moe_debug_kernel_launches(index: i32) -> i64;
     pub fn mi_moe_debug_plan_forward(cfg: *const mi_moe_config, T: i64, out: *mut c_char, cap: usize) -> c_int;
     pub fn mi_moe_debug_plan_grouped(N: i32, K: i32, bits: i32, glu: i32, total_rows: i64, max_active: i32, max_rows_per_expert: i64, max_streamed_rows: i64, tile_lists: i32, paired_out: i32, out: *mut c_char, cap: usize) -> c_int;
+    pub fn mi_moe_debug_tile_rule(cfg: *const mi_moe_config, T: i64, tiled: *mut i32, tile_min_rows: *mut i32) -> c_int;
     pub fn mi_moe_debug_side_streams_created() -> i32;
 
     pub fn mi_moe_stream_probe(buf: *const c_void, bytes: usize, sink: *mut u32, stream: *mut c_void) -> c_int;

@@ -112,14 +112,9 @@ def _check_against_fp64(blk, cfg, x, dbg, pick, got_bits, oracle_bits, what):
 
 def _plan(cfg, T):
     """Which segments the block tiles at this batch size: (tile lists built, rows from which a segment
-    is tiled).  The library's rule (csrc/common.hpp: tiled_batch, heavy_batch, tile_min_rows)."""
-    P, E = T * cfg.top_k, cfg.n_experts
-    light, heavy_avg = (6, 20) if cfg.bits == 4 else (17, 17)
-    even_groups = (cfg.hidden // 64) % 2 == 0 and (cfg.intermediate // 64) % 2 == 0
-    heavy = P >= heavy_avg * E
-    tiled = even_groups and (P >= light * E or heavy)
-    tmr = (9 if heavy else 17) if cfg.bits == 4 else 17
-    return tiled, tmr
+    is tiled): the library's own rule."""
+    import mlx_rs_amd as m
+    return m.capi.tile_rule(cfg.c_struct(), T)
 
 
 def _pair_classes(idx, counts, offsets, inv, tiled, tmr):

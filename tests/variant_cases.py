@@ -80,15 +80,9 @@ OP_CASE = dict(N=48, K=128, bits=4, rows=12, variant="qmm_small_kernel<4,0,1,0,0
 
 
 def rules(H, I, E, k, T, bits):
-    """(tile lists are built, rows from which a segment is tiled): the library's rule
-    (csrc/common.hpp: tiled_batch, heavy_batch, tile_min_rows)."""
-    P = T * k
-    light, heavy_avg = (6, 20) if bits == 4 else (17, 17)
-    even = (H // 64) % 2 == 0 and (I // 64) % 2 == 0
-    heavy = P >= heavy_avg * E
-    tiled = even and (P >= light * E or heavy)
-    tmr = (9 if (heavy and tiled) else 17) if bits == 4 else 17
-    return tiled, tmr
+    """(tile lists are built, rows from which a segment is tiled): the library's own rule."""
+    from mlx_rs_amd import capi
+    return capi.tile_rule(capi.Config(H, E, k, I, bits, 64, 0), T)
 
 
 def kernels_with_rows(plan, counts, T, tiled, tmr):
@@ -97,20 +91,12 @@ def kernels_with_rows(plan, counts, T, tiled, tmr):
     `counts` (rows per expert)."""
     classes = [c for c in (0, 1, 2) if (c == 0 and T > 128) or (c == 1 and T > 64) or c == 2]
     has = {0: False, 1: False, 2: False, "streamed": False}
+    from mlx_rs_amd import capi
     for c in counts:
-        c = int(c)
-        if c == 0:
-            continue
-        if not tiled or c < tmr:
-            has["streamed"] = True
-            continue
-        full, r = divmod(c, 256)
-        if full or r > 128:
-            has[0] = True
-        if 64 < r <= 128:
-            has[1] = True
-        if 0 < r <= 64:
-            has[2] = True
+        rows = capi.segment_rows_by_kernel(c, tiled, tmr)
+        for key, n in zip((0, 1, 2, "streamed"), rows):
+            if n:
+                has[key] = True
     names, product = set(), []
     for n in plan:
         product.append(n)

@@ -181,6 +181,17 @@ int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *route
                  int32_t score_mode, uint32_t *topk_idx, uint16_t *topk_w,
                  uint16_t *logits_out, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- R1 alone: logits = x . router_w^T (+ router_bias), bf16 [T, n_experts]: the gate Linear
+ * (mlx_matmul through nn::Linear, mlx-rs/src/nn/linear.rs:84-96, ops/arithmetic.rs:577-603), the way
+ * mi_moe_forward computes it: exact bf16 x bf16 products, summed without rounding, then fp64 -> fp32 ->
+ * bf16.  Up to 64 tokens in fp64 arithmetic; beyond, in integer arithmetic on the int8 matrix cores with
+ * the same bits (csrc/router_exact.hip), which needs workspace >= mi_moe_router_logits_workspace_size
+ * (contents irrelevant).  mi_moe_route keeps the fp64 route for any T and needs no such workspace. ---- */
+int mi_moe_router_logits_workspace_size(int64_t T, int32_t hidden, int32_t n_experts, size_t *bytes);
+int mi_moe_router_logits(const uint16_t *x, const uint16_t *router_w, const float *router_bias,
+                         int64_t T, int32_t hidden, int32_t n_experts, uint16_t *logits,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- R5 dispatch: stable sort of the P = T*k pairs by expert (mlx_argsort x2,
  * mlx_floor_divide, mlx_take; mlx-rs/src/ops/sort.rs:75-109).  Every output except
  * perm may be NULL.  workspace >= mi_moe_dispatch_workspace_size. */

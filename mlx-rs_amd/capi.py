@@ -30,6 +30,7 @@ EXPORTS = (
     "mi_moe_quantized_linear_typed", "mi_moe_dequantize_native",
     "mi_moe_debug_kernel_count", "mi_moe_debug_kernel_name", "mi_moe_debug_kernel_launches", "mi_moe_debug_plan_forward", "mi_moe_debug_plan_grouped",
     "mi_moe_debug_side_streams_created", "mi_moe_debug_tile_rule",
+    "mi_moe_router_logits_workspace_size", "mi_moe_router_logits",
 )
 
 
@@ -99,6 +100,8 @@ def load_library():
         "mi_moe_rms_norm": [vp, vp, C.c_float, i64, i32, vp, vp],
         "mi_moe_route_workspace_size": [i32, i64, C.POINTER(sz)],
         "mi_moe_route": [vp, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp, vp, sz, vp],
+        "mi_moe_router_logits_workspace_size": [i64, i32, i32, C.POINTER(sz)],
+        "mi_moe_router_logits": [vp, vp, vp, i64, i32, i32, vp, vp, sz, vp],
         "mi_moe_dispatch_workspace_size": [i32, i64, C.POINTER(sz)],
         "mi_moe_dispatch": [vp, i64, i32, vp, vp, vp, vp, vp, sz, vp],
         "mi_moe_gather_qmm_workspace_size": [i32, i64, i32, C.POINTER(sz)],

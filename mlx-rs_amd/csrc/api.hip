@@ -127,6 +127,8 @@ struct ForwardWs {
   void *disp_scratch;
   uint16_t *hh, *y, *xperm, *xnorm;
   uint16_t *gu;  // plain products only: the gate and the up product, [P, I] each
+  void *router_scratch;  // byte planes of x and of the router matrix (logits on the int8 matrix cores), or nullptr
+  size_t bytes_min;      // without the byte planes: a workspace of this size makes the forward take the fp64 logits (same bits)
   size_t bytes;
 };
 
@@ -159,6 +161,10 @@ ForwardWs carve_forward(const mi_moe_config &c, int64_t T, void *ws) {
   f.xperm = cv.take<uint16_t>(f.tiled && c.bits == 4 ? (size_t)T * c.hidden : 0);
   f.xnorm = cv.take<uint16_t>((size_t)T * c.hidden);  // rms_norm(x) of the residual variant
   f.gu = cv.take<uint16_t>(plain_config(c) ? 2 * (size_t)P * c.intermediate : 0);
+  f.bytes_min = cv.off;
+  const bool i8_router = router_logits_i8_applies(T, c.hidden, c.n_experts);  // (the last region: optional, see bytes_min)
+  f.router_scratch = cv.take<char>(i8_router ? router_logits_i8_bytes(T, c.hidden, c.n_experts) : 0);
+  if (!i8_router) f.router_scratch = nullptr;
   f.bytes = cv.off;
   return f;
 }
@@ -355,9 +361,10 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
   if (P > (int64_t)1 << 30) return fail("forward: too many (token, expert) pairs");
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u))
     return fail("forward: workspace must be non-NULL and 256-byte aligned");
-  const ForwardWs f = carve_forward(c, T, workspace);
-  if (workspace_bytes < f.bytes)
+  ForwardWs f = carve_forward(c, T, workspace);
+  if (workspace_bytes < f.bytes_min)
     return fail("forward: workspace too small (%zu bytes, need %zu)", workspace_bytes, f.bytes);
+  if (workspace_bytes < f.bytes) f.router_scratch = nullptr;  // room for everything but the byte planes: fp64 logits, same bits
   int stage = 0;
 #define MI_STAGE_DONE()                                  \
   do {                                                   \
@@ -388,8 +395,12 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     MI_STAGE_DONE();
     MI_STAGE_DONE();
   } else {
-    MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st,
-                                pair_in_router ? f.xperm : nullptr));
+    if (f.router_scratch)
+      MI_HIP(launch_router_logits_i8(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits,
+                                     f.router_scratch, st, pair_in_router ? f.xperm : nullptr));
+    else
+      MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st,
+                                  pair_in_router ? f.xperm : nullptr));
     MI_STAGE_DONE();
     MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
     MI_STAGE_DONE();
@@ -555,7 +566,7 @@ int mi_moe_forward_static(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_
   if (!h) return fail("forward_static: handle is NULL");
   if (T < 0) return fail("forward_static: negative token count");
   if (T * (int64_t)h->cfg.top_k > (int64_t)1 << 30) return fail("forward_static: too many (token, expert) pairs");
-  const size_t need = carve_forward(h->cfg, T, nullptr).bytes;
+  const size_t need = carve_forward(h->cfg, T, nullptr).bytes_min;
   if (need > (size_t)MI_MOE_STATIC_SCRATCH_BYTES)
     return fail("forward_static: %lld tokens of this layer need %zu bytes of workspace, the built-in scratch holds %zu "
                 "(use mi_moe_forward with a workspace of the caller's)",
@@ -659,6 +670,33 @@ int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *route
   MI_HIP(launch_router_select(logits, T, n_experts, top_k, score_mode, topk_idx, topk_w, st));
   return 0;
 } MI_CATCH("route")
+
+int mi_moe_router_logits_workspace_size(int64_t T, int32_t hidden, int32_t n_experts, size_t *bytes) try {
+  if (!bytes) return fail("router_logits_workspace_size: bytes is NULL");
+  if (T < 0 || hidden <= 0 || n_experts < 1 || n_experts > 512) return fail("router_logits_workspace_size: bad arguments");
+  *bytes = router_logits_i8_applies(T, hidden, n_experts) ? router_logits_i8_bytes(T, hidden, n_experts) + 256 : 256;
+  return 0;
+} MI_CATCH("router_logits_workspace_size")
+
+int mi_moe_router_logits(const uint16_t *x, const uint16_t *router_w, const float *router_bias, int64_t T,
+                         int32_t hidden, int32_t n_experts, uint16_t *logits, void *workspace,
+                         size_t workspace_bytes, void *stream) try {
+  if (T < 0) return fail("router_logits: negative token count");
+  if (hidden <= 0 || hidden % 64) return fail("router_logits: hidden must be a positive multiple of 64, got %d", hidden);
+  if (n_experts < 1 || n_experts > 512) return fail("router_logits: n_experts must be in [1, 512], got %d", n_experts);
+  if (T == 0) return 0;
+  if (!x || !router_w || !logits) return fail("router_logits: x, router_w and logits must be non-NULL");
+  if (!aligned16(x) || !aligned16(router_w)) return fail("router_logits: x and router_w must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (router_logits_i8_applies(T, hidden, n_experts)) {
+    const size_t need = router_logits_i8_bytes(T, hidden, n_experts) + 256;
+    if (!workspace || workspace_bytes < need) return fail("router_logits: workspace too small (need %zu bytes)", need);
+    MI_HIP(launch_router_logits_i8(x, router_w, router_bias, T, hidden, n_experts, logits, workspace, st));
+  } else {
+    MI_HIP(launch_router_logits(x, router_w, router_bias, T, hidden, n_experts, logits, st));
+  }
+  return 0;
+} MI_CATCH("router_logits")
 
 int mi_moe_dispatch_workspace_size(int32_t n_experts, int64_t P, size_t *bytes) try {
   if (!bytes) return fail("dispatch_workspace_size: bytes is NULL");

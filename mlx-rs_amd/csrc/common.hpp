@@ -268,6 +268,12 @@ bool router_logits_pairs_rows(int64_t T, int H);
 hipError_t launch_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,
                                 int64_t T, int H, int E, uint16_t *logits, hipStream_t st,
                                 uint16_t *x_paired = nullptr);
+// the same logits (bit for bit) on the int8 matrix cores, for prefill-sized batches: router_exact.hip.
+// scratch: router_logits_i8_bytes(T, H, E) bytes, contents irrelevant.
+bool router_logits_i8_applies(int64_t T, int H, int E);
+size_t router_logits_i8_bytes(int64_t T, int H, int E);
+hipError_t launch_router_logits_i8(const uint16_t *x, const uint16_t *wg, const float *bias, int64_t T, int H, int E,
+                                   uint16_t *logits, void *scratch, hipStream_t st, uint16_t *x_paired = nullptr);
 hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k, int mode,
                                 uint32_t *topk_idx, uint16_t *topk_w, hipStream_t st);
 size_t dispatch_workspace_bytes(int E, int64_t P);

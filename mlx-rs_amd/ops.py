@@ -238,6 +238,26 @@ def rms_norm(x, weight, eps=1e-5):
     return out.reshape(x.shape)
 
 
+def router_logits(x, router_w, router_bias=None):
+    """The gate Linear alone: bf16 logits [T, E] = x . router_w^T (+ router_bias), the way the block computes
+    them (mi_moe_router_logits: above 64 tokens on the int8 matrix cores, with the bits of the fp64 route)."""
+    lib = load_library()
+    _need(x, torch.bfloat16, "x")
+    _need(router_w, torch.bfloat16, "router_w")
+    T, H = x.shape
+    E = router_w.shape[0]
+    if router_w.shape[1] != H:
+        raise capi.MoeError(f"router_logits: x has {H} columns, router_w {router_w.shape[1]}")
+    logits = torch.empty((T, E), dtype=torch.bfloat16, device=x.device)
+    need = C.c_size_t()
+    check(lib.mi_moe_router_logits_workspace_size(T, H, E, C.byref(need)))
+    ws = _workspace(need.value, x.device)
+    check(lib.mi_moe_router_logits(_ptr(x), _ptr(router_w),
+                                   _ptr(None if router_bias is None else _need(router_bias, torch.float32, "router_bias")),
+                                   T, H, E, _ptr(logits), _ptr(ws), ws.numel(), _stream()))
+    return logits
+
+
 def route(x, router_w, top_k, score_mode=capi.SCORE_SOFTMAX_THEN_TOPK_RENORM, router_bias=None,
           return_logits=False):
     """Gate Linear + softmax(precise) + top-k + scores in one call (what an mlx-lm MoE block

@@ -80,6 +80,9 @@ extern "C" {
     pub fn mi_moe_route_workspace_size(n_experts: i32, T: i64, bytes: *mut usize) -> c_int;
     pub fn mi_moe_route(x: *const u16, router_w: *const u16, router_bias: *const f32, T: i64, hidden: i32, n_experts: i32, top_k: i32, score_mode: i32, topk_idx: *mut u32, topk_w: *mut u16, logits_out: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
 
+    pub fn mi_moe_router_logits_workspace_size(T: i64, hidden: i32, n_experts: i32, bytes: *mut usize) -> c_int;
+    pub fn mi_moe_router_logits(x: *const u16, router_w: *const u16, router_bias: *const f32, T: i64, hidden: i32, n_experts: i32, logits: *mut u16, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
+
     pub fn mi_moe_dispatch_workspace_size(n_experts: i32, P: i64, bytes: *mut usize) -> c_int;
     pub fn mi_moe_dispatch(expert_of_pair: *const u32, P: i64, n_experts: i32, counts: *mut u32, offsets: *mut u32, perm: *mut u32, inv_perm: *mut u32, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void) -> c_int;
 

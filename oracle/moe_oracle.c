@@ -215,7 +215,9 @@ void orc_router_logits(const uint16_t *x, const uint16_t *wg, const float *bias,
     for (int e = 0; e < E; ++e) {
       double acc = 0.0;
       const uint16_t *xr = x + t * H, *wr = wg + (int64_t)e * H;
-      for (int h = 0; h < H; ++h) acc += (double)(orc_bf16_to_f32(xr[h]) * orc_bf16_to_f32(wr[h]));
+      /* the product of two bf16 values is exact in double over the whole range (in float it would
+       * underflow below 2^-149: two factors of 1e-25 each) */
+      for (int h = 0; h < H; ++h) acc += (double)orc_bf16_to_f32(xr[h]) * (double)orc_bf16_to_f32(wr[h]);
       if (bias) acc += (double)bias[e];
       g[t * E + e] = orc_f32_to_bf16((float)acc);
     }

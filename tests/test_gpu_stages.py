@@ -250,3 +250,75 @@ def test_stream_probe_runs_and_rejects_bad_sizes():
     assert lib.mi_moe_stream_probe(buf.data_ptr(), 1000, sink.data_ptr(), st) != 0
     assert "32768" in m.capi.last_error()
     assert lib.mi_moe_stream_probe(None, 32768, sink.data_ptr(), st) != 0
+
+
+def _exact_logits_f64(x_bits, w_bits, bias):
+    """The definition the oracle and both device routes share, in numpy: exact products, float64 sums,
+    float64 -> float32 -> bfloat16 (pins orc.router_logits from outside, on the data of these tests)."""
+    from helpers import f32_of_bits
+    s = f32_of_bits(x_bits).astype(np.float64) @ f32_of_bits(w_bits).astype(np.float64).T
+    if bias is not None:
+        s = s + bias.astype(np.float64)
+    return s.astype(np.float32)
+
+
+@pytest.mark.parametrize("T,H,E,bias,kind", [
+    (65, 64, 1, False, "normal"), (100, 256, 8, True, "normal"), (128, 2048, 128, False, "normal"),
+    (333, 4096, 200, True, "normal"), (4096, 2048, 128, True, "normal"), (97, 1024, 512, False, "normal"),
+    # rows whose elements span 40 binades: many elements lose bits in fixed point, the bound sends their logits to fp64
+    (200, 512, 64, True, "wide"),
+    # rows of zeros, subnormals, values near the ends of the bfloat16 range, logits that cancel to (almost) nothing
+    (130, 256, 40, False, "edge"),
+    # infinities and NaNs in x and in the router matrix
+    (70, 128, 16, False, "nonfinite"),
+])
+def test_router_logits_on_the_int8_matrix_cores_have_the_fp64_bits(orc, m, T, H, E, bias, kind):
+    """mi_moe_router_logits above 64 tokens (integer arithmetic + a checked error bound + fp64 where the bound does
+    not decide) against the oracle's fp64 accumulation, bit for bit."""
+    print(f"router logits T={T} H={H} E={E} bias={bias} {kind}", flush=True)
+    rng = np.random.default_rng(T * 7 + E)
+    xf = rng.normal(0, 1, (T, H)).astype(np.float32)
+    wf = rng.normal(0, 0.02, (E, H)).astype(np.float32)
+    if kind == "wide":
+        xf *= np.exp2(rng.integers(-40, 1, (T, H))).astype(np.float32)
+        wf *= np.exp2(rng.integers(-30, 1, (E, H))).astype(np.float32)
+    if kind == "edge":
+        xf[0] = 0.0                                   # a token of zeros
+        xf[1] = 1e-40                                 # subnormal bfloat16 values
+        xf[2] = rng.normal(0, 1, H) * 1e-30
+        xf[3] = rng.normal(0, 1, H) * 1e18
+        xf[4, : H // 2] = 1.0
+        xf[4, H // 2:] = -1.0                         # against a constant router row: exact cancellation
+        xf[5] = xf[4]
+        xf[5, 0] = 1.0 + 2.0 ** -7                    # ... and cancellation down to one last place
+        wf[0] = 0.5
+        wf[1] = 0.0
+        wf[2] = rng.normal(0, 1, H) * 1e-25
+        wf[3] = rng.normal(0, 1, H) * 1e15
+        wf[4, ::2] = 1e-38
+    x, w = orc.f32_to_bf16(xf), orc.f32_to_bf16(wf)
+    if kind == "nonfinite":
+        x[3, 5] = 0x7F80   # +inf
+        x[9, 0] = 0x7FC0   # NaN
+        w[2, 7] = 0xFF80   # -inf
+    b = rng.normal(0, 1, E).astype(np.float32) if bias else None
+    got = bits_u16(m.ops.router_logits(bf16_tensor(x, "cuda"), bf16_tensor(w, "cuda"),
+                                       None if b is None else torch.from_numpy(b).cuda()))
+    torch.cuda.synchronize()
+    ref = orc.router_logits(x, w, b)
+    if kind == "nonfinite":
+        from helpers import f32_of_bits
+        g, r = f32_of_bits(got), f32_of_bits(ref)
+        assert np.array_equal(np.isnan(g), np.isnan(r)) and np.isnan(r).any()
+        ok = ~np.isnan(r)
+        assert np.array_equal(got[ok], ref[ok])
+        return
+    bad = np.argwhere(got != ref)
+    assert len(bad) == 0, (f"{len(bad)} of {got.size} logits differ from the fp64 accumulation; first (token, expert, got, oracle): "
+                           f"{[(int(t), int(e), hex(got[t, e]), hex(ref[t, e])) for t, e in bad[:8]]}")
+    if kind == "normal" and T * E * H <= 2 ** 28:
+        assert np.array_equal(orc.f32_to_bf16(_exact_logits_f64(x, w, b)), ref), "the oracle itself against numpy float64"
+    # the fp64 route (mi_moe_route's) gives the same bits
+    _, _, gl = m.ops.route(bf16_tensor(x, "cuda"), bf16_tensor(w, "cuda"), 1, 0,
+                           None if b is None else torch.from_numpy(b).cuda(), return_logits=True)
+    assert np.array_equal(bits_u16(gl), ref)

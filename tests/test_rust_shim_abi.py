@@ -94,7 +94,7 @@ def parse_rust():
 def test_every_header_function_is_declared_identically():
     hf, _, _ = parse_header()
     rf, _, _ = parse_rust()
-    assert len(hf) == 37, sorted(hf)
+    assert len(hf) == 39, sorted(hf)
     assert sorted(hf) == sorted(rf)
     for name, (ret, args) in hf.items():
         assert rf[name][0] == ret, (name, rf[name][0], ret)

@@ -51,8 +51,10 @@ def test_static_scratch_refuses_what_does_not_fit(orc):
     H, E, k, I = 2048, 128, 8, 768
     W = host_layer(orc, H, E, k, I, 4, seed=5)
     blk = device_block(m, m.MoeConfig(H, E, k, I), W)
-    T = 157  # one token more than 8 MiB of workspace serve for this layer
-    assert blk.workspace_bytes(T) - 256 > m.capi.STATIC_SCRATCH_BYTES >= blk.workspace_bytes(T - 1) - 256
+    T = 157  # one token more than 8 MiB of workspace serve for this layer (without the optional byte planes of the
+             # int8 router logits, which mi_moe_workspace_size counts in: on the built-in scratch the logits of a batch
+             # of more than 64 tokens come from the fp64 kernels, with the same bits)
+    assert blk.workspace_bytes(T) - 256 > m.capi.STATIC_SCRATCH_BYTES
     x = bf16_tensor(host_tokens(orc, T, H, seed=1), "cuda")
     out = torch.full_like(x, 7.0)
     st = torch.cuda.current_stream().cuda_stream

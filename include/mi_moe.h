@@ -174,7 +174,9 @@ int mi_moe_forward_timed(mi_moe_handle h, const uint16_t *x, int64_t T, uint16_t
  * take_along_axis + renormalise (mlx_matmul, mlx_softmax_axis, mlx_argpartition_axis,
  * mlx_take_along_axis, mlx_sum_axis, mlx_divide; mlx-rs/src/ops/arithmetic.rs:577-603,
  * 1291-1327, ops/sort.rs:211-260, ops/indexing/mod.rs:433-453).
- * logits_out (bf16 [T,E]) may be NULL.  workspace >= mi_moe_route_workspace_size. */
+ * logits_out (bf16 [T,E]) may be NULL.  workspace >= mi_moe_route_workspace_size.  A workspace that is larger
+ * by mi_moe_router_logits_workspace_size(T, hidden, n_experts) lets batches of more than 64 tokens take the
+ * integer route for the logits (same bits; up to 128 experts with the selection in the same kernel). */
 int mi_moe_route_workspace_size(int32_t n_experts, int64_t T, size_t *bytes);
 int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *router_bias,
                  int64_t T, int32_t hidden, int32_t n_experts, int32_t top_k,

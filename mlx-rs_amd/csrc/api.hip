@@ -395,15 +395,29 @@ static int forward_impl(mi_moe_handle h, const uint16_t *x_in, int64_t T, uint16
     MI_STAGE_DONE();
     MI_STAGE_DONE();
   } else {
-    if (f.router_scratch)
-      MI_HIP(launch_router_logits_i8(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits,
-                                     f.router_scratch, st, pair_in_router ? f.xperm : nullptr));
-    else
-      MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st,
-                                  pair_in_router ? f.xperm : nullptr));
-    MI_STAGE_DONE();
-    MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
-    MI_STAGE_DONE();
+    // Which route the logits take (all three give the same bits).  Measured, 128 experts, hidden 2048, logits +
+    // selection, us at 1024 / 2048 / 4096 / 8192 tokens: fp64 matrix cores 19.9 / 27.0 / 45.7 / 81.6; byte planes +
+    // int8 product, selection apart 22.5 / 26.5 / 39.7 / 64.1; one kernel per 32 tokens (planes in LDS, selection
+    // included; a block's phases follow each other, and there are T / 32 blocks) 41.3 / 41.9 / 45.2 / 49.5.
+    const int64_t logit_work = T * (int64_t)c.hidden * ((c.n_experts + 127) / 128);
+    const bool i8_pays = f.router_scratch && logit_work >= (int64_t)3 << 20;
+    if (i8_pays && logit_work >= (int64_t)12 << 20 && router_tile_applies(T, c.hidden, c.n_experts, c.top_k)) {
+      // logits and selection in one kernel (the stage times both land in the first)
+      MI_HIP(launch_router_tile(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, c.top_k, c.score_mode,
+                                f.logits, f.topk_idx, f.topk_w, f.router_scratch, st, pair_in_router ? f.xperm : nullptr));
+      MI_STAGE_DONE();
+      MI_STAGE_DONE();
+    } else {
+      if (i8_pays)
+        MI_HIP(launch_router_logits_i8(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits,
+                                       f.router_scratch, st, pair_in_router ? f.xperm : nullptr));
+      else
+        MI_HIP(launch_router_logits(x, h->w.router_w, h->w.router_bias, T, c.hidden, c.n_experts, f.logits, st,
+                                    pair_in_router ? f.xperm : nullptr));
+      MI_STAGE_DONE();
+      MI_HIP(launch_router_select(f.logits, T, c.n_experts, c.top_k, c.score_mode, f.topk_idx, f.topk_w, st));
+      MI_STAGE_DONE();
+    }
     MI_HIP(launch_dispatch(f.topk_idx, P, c.n_experts, c.top_k, f.counts, f.offsets, f.perm, f.inv_perm,
                            f.src_of, f.work, f.tiled ? f.mtiles : nullptr, f.max_mtiles, f.tmr,
                            f.disp_scratch, st));
@@ -666,7 +680,18 @@ int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *route
     logits = static_cast<uint16_t *>(workspace);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  MI_HIP(launch_router_logits(x, router_w, router_bias, T, hidden, n_experts, logits, st));
+  // with room for them behind the logits, the byte planes of the integer route (same bits, see mi_moe_router_logits)
+  const size_t lbytes = logits_out ? 0 : align_up((size_t)T * n_experts * 2);
+  void *planes = workspace ? static_cast<char *>(workspace) + lbytes : nullptr;
+  const bool roomy = workspace && router_logits_i8_applies(T, hidden, n_experts) &&
+                     workspace_bytes >= lbytes + router_logits_i8_bytes(T, hidden, n_experts) + 256;
+  if (roomy && router_tile_applies(T, hidden, n_experts, top_k)) {
+    MI_HIP(launch_router_tile(x, router_w, router_bias, T, hidden, n_experts, top_k, score_mode, logits, topk_idx, topk_w,
+                              planes, st));
+    return 0;
+  }
+  if (roomy) MI_HIP(launch_router_logits_i8(x, router_w, router_bias, T, hidden, n_experts, logits, planes, st));
+  else MI_HIP(launch_router_logits(x, router_w, router_bias, T, hidden, n_experts, logits, st));
   MI_HIP(launch_router_select(logits, T, n_experts, top_k, score_mode, topk_idx, topk_w, st));
   return 0;
 } MI_CATCH("route")

@@ -274,6 +274,11 @@ bool router_logits_i8_applies(int64_t T, int H, int E);
 size_t router_logits_i8_bytes(int64_t T, int H, int E);
 hipError_t launch_router_logits_i8(const uint16_t *x, const uint16_t *wg, const float *bias, int64_t T, int H, int E,
                                    uint16_t *logits, void *scratch, hipStream_t st, uint16_t *x_paired = nullptr);
+// logits and selection in one kernel, up to 128 experts (router_exact.hip); scratch as for launch_router_logits_i8
+bool router_tile_applies(int64_t T, int H, int E, int k);
+hipError_t launch_router_tile(const uint16_t *x, const uint16_t *wg, const float *bias, int64_t T, int H, int E, int k,
+                              int mode, uint16_t *logits, uint32_t *topk_idx, uint16_t *topk_w, void *scratch,
+                              hipStream_t st, uint16_t *x_paired = nullptr);
 hipError_t launch_router_select(const uint16_t *logits, int64_t T, int E, int k, int mode,
                                 uint32_t *topk_idx, uint16_t *topk_w, hipStream_t st);
 size_t dispatch_workspace_bytes(int E, int64_t P);

@@ -271,9 +271,12 @@ def route(x, router_w, top_k, score_mode=capi.SCORE_SOFTMAX_THEN_TOPK_RENORM, ro
     inds = torch.empty((T, top_k), dtype=torch.int32, device=x.device)
     sc = torch.empty((T, top_k), dtype=torch.bfloat16, device=x.device)
     logits = torch.empty((T, E), dtype=torch.bfloat16, device=x.device)
+    need = C.c_size_t()
+    check(lib.mi_moe_router_logits_workspace_size(T, H, E, C.byref(need)))  # room for the integer route's byte planes
+    ws = _workspace(need.value + 256, x.device)
     check(lib.mi_moe_route(_ptr(x), _ptr(router_w),
                            _ptr(None if router_bias is None else _need(router_bias, torch.float32, "router_bias")),
-                           T, H, E, top_k, score_mode, _ptr(inds), _ptr(sc), _ptr(logits), None, 0, _stream()))
+                           T, H, E, top_k, score_mode, _ptr(inds), _ptr(sc), _ptr(logits), _ptr(ws), ws.numel(), _stream()))
     return (inds, sc, logits) if return_logits else (inds, sc)
 
 

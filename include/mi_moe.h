@@ -188,7 +188,8 @@ int mi_moe_route(const uint16_t *x, const uint16_t *router_w, const float *route
  * mi_moe_forward computes it: exact bf16 x bf16 products, summed without rounding, then fp64 -> fp32 ->
  * bf16.  Up to 64 tokens in fp64 arithmetic; beyond, in integer arithmetic on the int8 matrix cores with
  * the same bits (csrc/router_exact.hip), which needs workspace >= mi_moe_router_logits_workspace_size
- * (contents irrelevant).  mi_moe_route keeps the fp64 route for any T and needs no such workspace. ---- */
+ * (contents irrelevant).  mi_moe_route takes the fp64 route for any T unless its workspace has that much
+ * room beyond its own need. ---- */
 int mi_moe_router_logits_workspace_size(int64_t T, int32_t hidden, int32_t n_experts, size_t *bytes);
 int mi_moe_router_logits(const uint16_t *x, const uint16_t *router_w, const float *router_bias,
                          int64_t T, int32_t hidden, int32_t n_experts, uint16_t *logits,

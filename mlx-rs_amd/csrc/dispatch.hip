@@ -39,62 +39,66 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_hist_kernel(
   for (int i = tid; i < E; i += kDispThreads) blockhist[(int64_t)blockIdx.x * E + i] = lds[i];
 }
 
-// Per-block histograms -> counts, offsets, records, M tiles, and each block's first sorted position per
-// expert.  The blocks are dealt in G = 1024 / E' contiguous ranges (E' = E rounded up to a power of
-// two) to G threads per expert, so that a thread walks nb / G histograms, not nb.
-__global__ __launch_bounds__(kDispThreads) void dispatch_scan_kernel(
-    uint32_t *__restrict__ blockhist, int nb, int E, uint32_t *__restrict__ counts,
-    uint32_t *__restrict__ offsets, uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles,
-    int cap256, uint32_t big_thr) {
+// Scatter of block b's pairs, and what used to be a kernel of its own between the histograms and the
+// scatter: every block sums the per-block histograms itself (nb x E words, a few loads per thread: the
+// blocks are dealt in G = 1024 / E' contiguous ranges, E' = E rounded up to a power of two, to G threads
+// per expert), which gives it the counts, their exclusive scan and the number of pairs of each expert in
+// the blocks before it, i.e. its own first sorted position per expert.  One more block (blockIdx.x == nb)
+// takes no pairs and writes counts, offsets, work records and M tiles instead.
+__global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
+    const uint32_t *flat, int64_t P, int E, int nbits, int k_div, int64_t span,
+    const uint32_t *__restrict__ blockhist, int nb, uint32_t *__restrict__ counts, uint32_t *__restrict__ offsets,
+    uint32_t *__restrict__ work, uint32_t *__restrict__ mtiles, int cap256, uint32_t big_thr,
+    uint32_t *__restrict__ perm, uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of) {
   extern __shared__ uint32_t lds[];
-  __shared__ uint32_t n_active;
-  uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *part = lds + 3 * E;  // part[G][E]
+  __shared__ uint32_t n_active, total;
+  uint32_t *cnt = lds, *tmp = lds + E, *cur = lds + 2 * E, *wcnt = lds + 3 * E;  // tmp: at least kDispWaves words
   const int tid = threadIdx.x;
+  const int mine = (int)blockIdx.x;
   int ep = 1;
   while (ep < E) ep <<= 1;
   const int G = kDispThreads / ep;  // E <= 512: at least 2
   const int e = tid % ep, g = tid / ep;
   const int per = (nb + G - 1) / G;
   const int b0 = g * per, b1 = b0 + per < nb ? b0 + per : nb;
+  uint32_t *part_all = wcnt, *part_before = wcnt + G * E;  // [G][E] each; the space is wcnt's afterwards
   if (e < E) {
-    uint32_t run = 0;
-    for (int b = b0; b < b1; ++b) run += blockhist[(int64_t)b * E + e];
-    part[g * E + e] = run;
-  }
-  __syncthreads();
-  if (tid < E) {
-    uint32_t run = 0;
-    for (int i = 0; i < G; ++i) run += part[i * E + tid];
-    cnt[tid] = run;
-  }
-  __syncthreads();
-  finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, cap256, big_thr, &n_active);
-  if (e < E) {  // blockhist[b][e] <- first sorted position of expert e for block b
-    uint32_t run = cur[e];
-    for (int i = 0; i < g; ++i) run += part[i * E + e];
+    uint32_t all = 0, before = 0;
     for (int b = b0; b < b1; ++b) {
-      uint32_t c = blockhist[(int64_t)b * E + e];
-      blockhist[(int64_t)b * E + e] = run;
-      run += c;
+      const uint32_t c = blockhist[(int64_t)b * E + e];
+      all += c;
+      before += b < mine ? c : 0u;
     }
+    part_all[g * E + e] = all;
+    part_before[g * E + e] = before;
   }
-}
-
-__global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
-    const uint32_t *flat, int64_t P, int E, int nbits, int k_div, int64_t span,
-    const uint32_t *__restrict__ blockbase, uint32_t *__restrict__ perm,
-    uint32_t *__restrict__ inv_perm, uint32_t *__restrict__ src_of) {
-  extern __shared__ uint32_t lds[];
-  uint32_t *cur = lds, *wcnt = lds + E;
-  const int tid = threadIdx.x;
-  for (int i = tid; i < E; i += kDispThreads) cur[i] = blockbase[(int64_t)blockIdx.x * E + i];
   __syncthreads();
-  const int64_t j0 = (int64_t)blockIdx.x * span;
+  uint32_t before = 0;
+  if (tid < E) {
+    uint32_t all = 0;
+    for (int i = 0; i < G; ++i) {
+      all += part_all[i * E + tid];
+      before += part_before[i * E + tid];
+    }
+    cnt[tid] = all;
+  }
+  __syncthreads();
+  if (mine == nb) {
+    finish_counts(cnt, tmp, cur, E, counts, offsets, work, mtiles, cap256, big_thr, &n_active);
+    return;
+  }
+  block_exclusive_scan(cnt, tmp, E, &total);
+  if (tid < E) cur[tid] = cnt[tid] + before;
+  __syncthreads();
+  const int64_t j0 = (int64_t)mine * span;
   const int64_t j1 = j0 + span < P ? j0 + span : P;
   scatter_range(flat, j0, j1, E, nbits, k_div, cur, wcnt, perm, inv_perm, src_of);
 }
 
-constexpr int64_t kSpan = 2048;  // pairs per block in the multi-block path
+#ifndef MI_DISPATCH_SPAN
+#define MI_DISPATCH_SPAN 1024
+#endif
+constexpr int64_t kSpan = MI_DISPATCH_SPAN;  // pairs per block in the multi-block path
 
 size_t dispatch_workspace_bytes(int E, int64_t P) {
   if (P <= kSingleMaxP) return 256;
@@ -118,10 +122,13 @@ hipError_t launch_dispatch(const uint32_t *flat, int64_t P, int E, int k_div, ui
   uint32_t *blockhist = reinterpret_cast<uint32_t *>(scratch);
   const int nb = (int)((P + kSpan - 1) / kSpan);
   dispatch_hist_kernel<<<nb, kDispThreads, (size_t)E * 4, st>>>(flat, P, E, kSpan, blockhist);
-  dispatch_scan_kernel<<<1, kDispThreads, ((size_t)3 * E + kDispThreads) * 4, st>>>(blockhist, nb, E, counts,
-                                                                  offsets, work, mtiles, cap256, (uint32_t)big_thr);
-  dispatch_scatter_kernel<<<nb, kDispThreads, (size_t)(1 + kDispWaves) * E * 4, st>>>(
-      flat, P, E, nbits, k_div, kSpan, blockhist, perm, inv_perm, src_of);
+  // LDS: cnt, tmp, cur [E] each (tmp also holds kDispWaves words), then the larger of wcnt[16 E] and the two
+  // partial-sum arrays [G][E] (G E <= 1024)
+  const size_t e3 = (size_t)3 * (E > kDispWaves ? E : kDispWaves);
+  const size_t tail = (size_t)kDispWaves * E > 2u * kDispThreads ? (size_t)kDispWaves * E : 2u * kDispThreads;
+  dispatch_scatter_kernel<<<nb + 1, kDispThreads, (e3 + tail) * 4, st>>>(flat, P, E, nbits, k_div, kSpan, blockhist, nb, counts,
+                                                                        offsets, work, mtiles, cap256, (uint32_t)big_thr, perm,
+                                                                        inv_perm, src_of);
   return hipGetLastError();
 }
 

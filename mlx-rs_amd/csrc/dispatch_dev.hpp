@@ -25,25 +25,26 @@ __device__ __forceinline__ uint64_t match_peers(uint32_t e, int nbits, bool vali
 }
 
 // exclusive scan of v[0..n) in LDS by one block of kDispThreads threads (n <= 1024);
-// tmp: n words.  Returns with v holding the exclusive scan and *total the sum.
+// tmp: at least kDispWaves words.  Returns with v holding the exclusive scan and *total the sum.
+// Each wave scans its 64 values with lane shuffles; the waves' totals meet in tmp.
 __device__ __forceinline__ void block_exclusive_scan(uint32_t *v, uint32_t *tmp, int n, uint32_t *total) {
-  const int tid = threadIdx.x;
-  uint32_t mine = tid < n ? v[tid] : 0u;
-  uint32_t *src = v, *dst = tmp;
-  for (int off = 1; off < n; off <<= 1) {
-    uint32_t val = 0;
-    if (tid < n) val = src[tid] + (tid >= off ? src[tid - off] : 0u);
-    __syncthreads();
-    if (tid < n) dst[tid] = val;
-    __syncthreads();
-    uint32_t *t = src;
-    src = dst;
-    dst = t;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const uint32_t mine = tid < n ? v[tid] : 0u;
+  uint32_t incl = mine;
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t up = __shfl_up(incl, d, kWave);
+    if (lane >= d) incl += up;
   }
-  uint32_t incl = tid < n ? src[tid] : 0u;
+  if (lane == kWave - 1) tmp[wave] = incl;
   __syncthreads();
-  if (tid < n) v[tid] = incl - mine;
-  if (tid == n - 1) *total = incl;
+  uint32_t before = 0, all = 0;
+  for (int w = 0; w < kDispWaves; ++w) {
+    const uint32_t t = tmp[w];
+    before += w < wave ? t : 0u;
+    all += t;
+  }
+  if (tid < n) v[tid] = before + incl - mine;
+  if (tid == 0) *total = all;
   __syncthreads();
 }
 

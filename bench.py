@@ -33,9 +33,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # scaled by what the same counters read for a plain copy kernel of known size.  Counters cannot be read from
 # inside this script: the figure is carried from the named file under profiles/, it is not measured by this run.
 CARRIED_TRAFFIC = {
-    "decode": (1.976e8, "profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt"),
-    "prefill": (4.049e8, "profiles/qmm_large_kernel_prefill_tokens4096_counters.txt"),
-    "mixtral_decode": (2.527e8, "profiles/qmm_small_kernel_decode_mixtral_batch1.txt"),
+    "decode": (1.975e8, "profiles/qmm_small_kernel_decode_batch32_hbm_traffic.txt"),
+    "prefill": (4.054e8, "profiles/qmm_large_kernel_prefill_tokens4096_counters.txt"),
+    "mixtral_decode": (2.528e8, "profiles/qmm_small_kernel_decode_mixtral_batch1.txt"),
 }
 
 WORKLOADS = {

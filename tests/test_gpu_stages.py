@@ -55,7 +55,10 @@ def test_route_ties_go_to_the_lower_expert(orc, m):
 
 
 @pytest.mark.parametrize("P,E", [(1, 8), (8, 128), (256, 128), (4096, 8), (4097, 128), (40000, 64), (70000, 500),
-                                 (1, 1), (300, 1), (5000, 1)])
+                                 (1, 1), (300, 1), (5000, 1),
+                                 # several blocks, each summing the others' histograms: expert counts that are
+                                 # not powers of two, the largest one, pair counts around the per-block span
+                                 (5000, 3), (9000, 33), (8193, 200), (20000, 512), (5120, 16), (5121, 16)])
 def test_dispatch_bit_exact(orc, m, P, E):
     print(f"dispatch P={P} E={E}", flush=True)
     rng = np.random.default_rng(P)

@@ -24,6 +24,15 @@
 #ifndef MI_MOE_WEAVE
 #define MI_MOE_WEAVE 1
 #endif
+// VALU instructions of the stage woven in after each MFMA of a step, per 32-row token sub-tile of a wave
+// (256-row tiles / shorter ones; measured: 16 / 12, with 12 / 12 the 256-row class loses 1 %, with 16 / 16 the
+// 128-row class 7 %)
+#ifndef MI_WEAVE_VALU
+#define MI_WEAVE_VALU 16
+#endif
+#ifndef MI_WEAVE_VALU_SHORT
+#define MI_WEAVE_VALU_SHORT 12
+#endif
 
 namespace mi_moe {
 
@@ -202,15 +211,20 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
     const float sc = (gi & 1) ? bf16hi_to_f32(sw) : bf16lo_to_f32(sw);
     float bi = (gi & 1) ? bf16hi_to_f32(bw) : bf16lo_to_f32(bw);
     if constexpr (BITS == 4) {
-      bi = __builtin_fmaf(-128.0f, sc, bi);  // codes are expanded as 128 + q
+      // codes are expanded as the fp16 values 1024 + q (exact: 0x6400 is 1024.0 with a last place of 1), a pair
+      // (q_i, q_{i+4}) per register in one shift and one and-or; the mixed-precision fma reads the halves as
+      // they are, so no conversion instruction stands between the codes and w_hat
+      typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+      bi = __builtin_fmaf(-1024.0f, sc, bi);
 #pragma unroll
       for (int wi = 0; wi < 2; ++wi) {
         const uint32_t w = R.bw[wi];
         uint32_t o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const uint32_t pr = ((w >> (4 * i)) & 0x000f000fu) | 0x43004300u;  // (128+q_i, 128+q_{i+4})
-          o[i] = cvt_pk_bf16(__builtin_fmaf(sc, bf16lo_to_f32(pr), bi), __builtin_fmaf(sc, bf16hi_to_f32(pr), bi));
+          const uint32_t pr = __builtin_amdgcn_bitop3_b32(w >> (4 * i), 0x000f000fu, 0x64006400u, 0xEA);  // (a & b) | c
+          const half2_t h = __builtin_bit_cast(half2_t, pr);
+          o[i] = cvt_pk_bf16(__builtin_fmaf(sc, (float)h.x, bi), __builtin_fmaf(sc, (float)h.y, bi));
         }
         Bt[tile_off(br, 2 * bh + wi)] = u32x4_t{o[0], o[1], o[2], o[3]};
       }
@@ -292,7 +306,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, MT 
 #pragma unroll
         for (int i = 0; i < 4 * MS; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 16 / MS, 0);  // its share of the stage's VALU work
+          __builtin_amdgcn_sched_group_barrier(0x002, (MT == 4 ? MI_WEAVE_VALU : MI_WEAVE_VALU_SHORT) / MS, 0);  // its share of the stage's VALU work
           if (i < 2 + MS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the remaining LDS reads
         }
       }
